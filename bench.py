@@ -821,7 +821,7 @@ def sobunex_leg(a, dev):
         wv, bv = torch.randn(W, device=dev), torch.randn(W, device=dev)
         ob, o32 = torch.empty(T, W, dtype=torch.bfloat16, device=dev), torch.empty(T, W, device=dev)
         t_new = timed(lambda: _call("mrs_hyb_layernorm", x, W, None, wv, bv, ob, o32, None, 0, T, W, 1e-6, 1), 10)
-        t_old = timed(lambda: _call("mrs_hyb_rmsnorm", x, W, wv, ob, o32, None, T, W, 1, 1e-6, 1, 1, None, 0), 10)
+        t_old = timed(lambda: _call("mrs_hyb_rmsnorm", x, W, wv, ob, o32, None, T, W, 1, 1e-6, 1, 1, None, 0, 0), 10)
         nb_ = T * W * (4 + 2 + 4)
         kern["norm_2048_rows"] = {"min_bytes": nb_, "sobunex_layernorm": {"us": round(1e6 * t_new, 1), "hbm_frac": round(nb_ / t_new / HBM_PEAK, 4)},
                                   "gekilix_rmsnorm": {"us": round(1e6 * t_old, 1), "hbm_frac": round(nb_ / t_old / HBM_PEAK, 4)}, "time_ratio": round(t_new / t_old, 2)}

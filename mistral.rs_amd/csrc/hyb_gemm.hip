@@ -25,7 +25,16 @@ struct GemmArgs {
   const int *bounds;         // grouped: [groups + 1] row bounds (device), else null
   long long wstride;         // elements between the groups' weight slabs
   int vec_ok;                // K, lda, ldw multiples of 8 (bf16) / 4 (f32) and 16-byte aligned bases: vector loads
+  // batched form (bounds null, batch > 0): blockIdx.z = b multiplies A + b * a_bstride with the slab W + b * wstride into C + b * c_bstride (per-head products: the
+  // heads' operands are column blocks of one row-major buffer)
+  int batch;
+  long long a_bstride, c_bstride;
+  int c_is_T;                // C holds T (bf16 | f32 as the operands), rounded once in the epilogue, instead of f32 (no accumulate then): the consumer is another product
 };
+template <class T> __device__ __forceinline__ void store_c(const GemmArgs &a, size_t idx, float v) {
+  if (a.c_is_T) ((T *)a.C)[idx] = from_f<T>(v);
+  else a.C[idx] = a.accumulate ? a.C[idx] + v : v;
+}
 
 constexpr int BM = 64, BN = 64, BK = 32;
 
@@ -80,6 +89,9 @@ __global__ void __launch_bounds__(256) gemm_tile_bf16_kernel(GemmArgs a) {
     row_hi = a.bounds[blockIdx.z + 1];
     W += (size_t)blockIdx.z * a.wstride;
   }
+  const bf16_t *A = (const bf16_t *)a.A;
+  size_t c_off = 0;
+  if (a.batch > 0) { A += (size_t)blockIdx.z * a.a_bstride; W += (size_t)blockIdx.z * a.wstride; c_off = (size_t)blockIdx.z * a.c_bstride; }
   const int m0 = row_lo + blockIdx.y * BM, n0 = blockIdx.x * BN;
   if (m0 >= row_hi) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ql = lane & 31, kh = lane >> 5;
@@ -88,7 +100,7 @@ __global__ void __launch_bounds__(256) gemm_tile_bf16_kernel(GemmArgs a) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.f;
   for (int k0 = 0; k0 < a.K; k0 += BK) {
-    TileLoad<bf16_t>::load((const bf16_t *)a.A, a.lda, m0, row_hi, k0, a.K, a.vec_ok, tid, As);
+    TileLoad<bf16_t>::load(A, a.lda, m0, row_hi, k0, a.K, a.vec_ok, tid, As);
     TileLoad<bf16_t>::load(W, a.ldw, n0, a.N, k0, a.K, a.vec_ok, tid, Ws);
     __syncthreads();
 #pragma unroll
@@ -106,10 +118,7 @@ __global__ void __launch_bounds__(256) gemm_tile_bf16_kernel(GemmArgs a) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int m = m0 + wm + (r & 3) + 8 * (r >> 2) + 4 * kh;
-      if (m < row_hi) {
-        float *c = a.C + (size_t)m * a.ldc + n;
-        *c = a.accumulate ? *c + acc[r] : acc[r];
-      }
+      if (m < row_hi) store_c<bf16_t>(a, c_off + (size_t)m * a.ldc + n, acc[r]);
     }
   }
 }
@@ -130,6 +139,8 @@ __global__ void __launch_bounds__(256) gemm_tile128_bf16_kernel(GemmArgs a) {
   const int m0 = row_lo + blockIdx.y * TM, n0 = blockIdx.x * TN;
   if (m0 >= row_hi) return;
   const bf16_t *A = (const bf16_t *)a.A;
+  size_t c_off = 0;
+  if (a.batch > 0) { A += (size_t)blockIdx.z * a.a_bstride; W += (size_t)blockIdx.z * a.wstride; c_off = (size_t)blockIdx.z * a.c_bstride; }
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, ql = lane & 31, kh = lane >> 5;
   const int wm = (wave & 1) * 64, wn = (wave >> 1) * 64;
   const int lr = tid >> 2, kc = (tid & 3) * 8;  // this thread stages rows lr and lr + 64 of both operands, 8 values at kc
@@ -189,10 +200,7 @@ __global__ void __launch_bounds__(256) gemm_tile128_bf16_kernel(GemmArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int m = m0 + wm + 32 * i + (r & 3) + 8 * (r >> 2) + 4 * kh;
-        if (m < row_hi) {
-          float *c = a.C + (size_t)m * a.ldc + n;
-          *c = a.accumulate ? *c + acc[i][j][r] : acc[i][j][r];
-        }
+        if (m < row_hi) store_c<bf16_t>(a, c_off + (size_t)m * a.ldc + n, acc[i][j][r]);
       }
   }
 }
@@ -207,6 +215,9 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
     row_hi = a.bounds[blockIdx.z + 1];
     W += (size_t)blockIdx.z * a.wstride;
   }
+  const float *A = (const float *)a.A;
+  size_t c_off = 0;
+  if (a.batch > 0) { A += (size_t)blockIdx.z * a.a_bstride; W += (size_t)blockIdx.z * a.wstride; c_off = (size_t)blockIdx.z * a.c_bstride; }
   const int m0 = row_lo + blockIdx.y * BM, n0 = blockIdx.x * BN;
   if (m0 >= row_hi) return;
   const int tid = threadIdx.x, tn = tid & 15, tm = tid >> 4;  // thread: rows tm + 16 i, columns tn + 16 j
@@ -216,7 +227,7 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
   for (int k0 = 0; k0 < a.K; k0 += BK) {
-    TileLoad<float>::load((const float *)a.A, a.lda, m0, row_hi, k0, a.K, a.vec_ok, tid, As);
+    TileLoad<float>::load(A, a.lda, m0, row_hi, k0, a.K, a.vec_ok, tid, As);
     TileLoad<float>::load(W, a.ldw, n0, a.N, k0, a.K, a.vec_ok, tid, Ws);
     __syncthreads();
 #pragma unroll
@@ -245,10 +256,7 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tn + 16 * j;
-      if (n < a.N) {
-        float *c = a.C + (size_t)m * a.ldc + n;
-        *c = a.accumulate ? *c + acc[i][j] : acc[i][j];
-      }
+      if (n < a.N) store_c<float>(a, c_off + (size_t)m * a.ldc + n, acc[i][j]);
     }
   }
 }
@@ -261,6 +269,7 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
 //              routed inputs)
 //   IN_GLU_CLAMP  A = f32 [M, 2 K] = gate | up: g = min(gate, p0), u = clamp(up, -p0, p0): x_k = round_T(g sigmoid(p1 g) (u + 1))
 //   IN_BIAS_XIELU A = f32 [M, K]: z = A + in_bias: x_k = round_T(z > 0 ? p0 z^2 + z / 2 : p1 (e^z - 1 - z) + z / 2)
+// The batched form offsets A by columns: only IN_PLAIN reads it there.
 enum { IN_PLAIN = 0, IN_GLU = 1, IN_SCALED = 2, IN_GLU_CLAMP = 3, IN_BIAS_XIELU = 4 };
 struct GemvArgs {
   const void *A;
@@ -276,6 +285,9 @@ struct GemvArgs {
   int src_div;
   const float *in_bias;      // IN_BIAS_XIELU
   float p0, p1;              // IN_GLU_CLAMP: limit, sigmoid factor; IN_BIAS_XIELU: the two coefficients
+  int batch;                 // batched form (row_group null): blockIdx.z = b reads A at column offset b * a_bstride, the slab W + b * wstride, writes C at column offset b * c_bstride
+  long long a_bstride, c_bstride;
+  int c_is_T;                // C holds T instead of f32 (no accumulate)
 };
 
 template <class T> struct Vec8;
@@ -309,7 +321,7 @@ __device__ __forceinline__ float xielu_in(float z, float ap, float an) { return 
 
 // one activation value (element path) / eight (vector path) of row m at column k, as the product sees it
 template <class T, int IN> __device__ __forceinline__ float act1(const GemvArgs &a, int m, int k) {
-  if (IN == IN_PLAIN) return to_f<T>(((const T *)a.A)[(size_t)m * a.lda + k]);
+  if (IN == IN_PLAIN) return to_f<T>(((const T *)a.A)[(size_t)blockIdx.z * a.a_bstride + (size_t)m * a.lda + k]);
   const float *A = (const float *)a.A;
   if (IN == IN_GLU) return round_to<T>(silu_in(A[(size_t)m * a.lda + k]) * A[(size_t)m * a.lda + a.K + k]);
   if (IN == IN_GLU_CLAMP) return round_to<T>(glu_clamp_in(A[(size_t)m * a.lda + k], A[(size_t)m * a.lda + a.K + k], a.p0, a.p1));
@@ -318,7 +330,7 @@ template <class T, int IN> __device__ __forceinline__ float act1(const GemvArgs 
   return round_to<T>((a.src_scale ? a.src_scale[r] : 1.0f) * A[(size_t)(r / a.src_div) * a.lda + k]);
 }
 template <class T, int IN> __device__ __forceinline__ void act8(const GemvArgs &a, int m, int k, float *x) {
-  if (IN == IN_PLAIN) { Vec8<T>::load((const T *)a.A + (size_t)m * a.lda + k, x); return; }
+  if (IN == IN_PLAIN) { Vec8<T>::load((const T *)a.A + (size_t)blockIdx.z * a.a_bstride + (size_t)m * a.lda + k, x); return; }
   const float *A = (const float *)a.A;
   if (IN == IN_GLU) {
     float g[8], u[8];
@@ -361,6 +373,8 @@ template <class T, int MR, int IN> __global__ void __launch_bounds__(256) gemv_r
     m_lo = blockIdx.y;
     m_cnt = 1;
     W += (size_t)a.row_group[m_lo] * a.wstride;
+  } else if (a.batch > 0) {
+    W += (size_t)blockIdx.z * a.wstride;
   }
   const T *wr = W + (size_t)n * a.ldw;
   float acc[MR];
@@ -391,8 +405,9 @@ template <class T, int MR, int IN> __global__ void __launch_bounds__(256) gemv_r
     if (m >= m_cnt) break;
     const float s = wave_sum(acc[m]);
     if (lane == 0) {
-      float *c = a.C + (size_t)(m_lo + m) * a.ldc + n;
-      *c = a.accumulate ? *c + s : s;
+      const size_t idx = (size_t)blockIdx.z * a.c_bstride + (size_t)(m_lo + m) * a.ldc + n;
+      if (a.c_is_T) ((T *)a.C)[idx] = from_f<T>(s);
+      else a.C[idx] = a.accumulate ? a.C[idx] + s : s;
     }
   }
 }
@@ -408,27 +423,57 @@ using namespace mrs::hyb;
 extern "C" const char *mrs_hyb_gemm_last_error() { return g_err; }
 
 // dtype: 1 bf16, 2 f32.  groups > 0: grouped form (bounds [groups + 1] on the device, max_rows = the largest number of rows a group can have).
-extern "C" int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
-                            const int *bounds, int groups, long long wstride, int max_rows, void *stream) {
+static int gemm_launch(const void *A, const void *W, void *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
+                       const int *bounds, int groups, long long wstride, int max_rows, int batch, long long a_bstride, long long c_bstride, int c_is_T, void *stream) {
   if (M <= 0 || N <= 0) return 0;
+  if (batch > 0 && groups > 0) return fail("mrs_hyb_gemm: grouped and batched at once");
+  if (c_is_T && accumulate) return fail("mrs_hyb_gemm: a product that writes operands does not accumulate");
+  if (batch > 65535) return fail("mrs_hyb_gemm: more than 65535 products in one batch");
   if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2)) return fail("mrs_hyb_gemm: bad shape / dtype");
   const int esz = dtype == 1 ? 2 : 4, vq = 8;
-  GemmArgs a{A, W, C, M, N, K, lda, ldw, ldc, accumulate, groups > 0 ? bounds : nullptr, wstride,
-             (K % vq == 0 && lda % vq == 0 && ldw % vq == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0) ? 1 : 0};
+  GemmArgs a{A, W, (float *)C, M, N, K, lda, ldw, ldc, accumulate, groups > 0 ? bounds : nullptr, wstride,
+             (K % vq == 0 && lda % vq == 0 && ldw % vq == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0 &&
+              (batch <= 0 || (a_bstride * esz) % 16 == 0)) ? 1 : 0, batch > 0 ? batch : 0, a_bstride, c_bstride, c_is_T};
+  const int gz = groups > 0 ? groups : (batch > 0 ? batch : 1);
   const int rows = groups > 0 ? max_rows : M;
   if (rows <= 0) return 0;
   // prompt-sized bf16 products take the 128 x 128 tile: dense from 256 rows, grouped when a group averages a full tile of rows
   if (dtype == 1 && N >= 128 && (groups > 0 ? M / groups >= 128 : M >= 256)) {
-    dim3 g2((N + 127) / 128, (rows + 127) / 128, groups > 0 ? groups : 1);
+    dim3 g2((N + 127) / 128, (rows + 127) / 128, gz);
     if (g2.y > 65535 || g2.z > 65535) return fail("mrs_hyb_gemm: too many row tiles / groups for one launch");
     hipLaunchKernelGGL(gemm_tile128_bf16_kernel, g2, dim3(256), 0, (hipStream_t)stream, a);
     return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm: launch failed");
   }
-  dim3 grid((N + BN - 1) / BN, (rows + BM - 1) / BM, groups > 0 ? groups : 1);
+  dim3 grid((N + BN - 1) / BN, (rows + BM - 1) / BM, gz);
   if (grid.y > 65535 || grid.z > 65535) return fail("mrs_hyb_gemm: too many row tiles / groups for one launch");
   if (dtype == 1) hipLaunchKernelGGL(gemm_tile_bf16_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
   else hipLaunchKernelGGL(gemm_tile_f32_kernel, grid, dim3(256), 0, (hipStream_t)stream, a);
   return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm: launch failed");
+}
+
+extern "C" int mrs_hyb_gemm(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate,
+                            const int *bounds, int groups, long long wstride, int max_rows, void *stream) {
+  return gemm_launch(A, W, C, M, N, K, lda, ldw, ldc, dtype, accumulate, bounds, groups, wstride, max_rows, 0, 0, 0, 0, stream);
+}
+/* `batch` products in one launch: product b multiplies A + b * a_bstride [M, K] (row stride lda) with W + b * wstride [N, K] into C + b * c_bstride (row stride ldc): the heads'
+ * operands as column blocks of row-major buffers.  c_is_T: C holds dtype values (rounded once) instead of f32.  batch 0: one product.  At most 8 rows take the row kernel. */
+extern "C" int mrs_hyb_gemm_batched(const void *A, const void *W, void *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int batch, long long a_bstride,
+                                    long long wstride, long long c_bstride, int c_is_T, void *stream) {
+  if (M <= 0 || N <= 0) return 0;
+  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2) || batch < 0) return fail("mrs_hyb_gemm_batched: bad shape / dtype");
+  if (M > 8) return gemm_launch(A, W, C, M, N, K, lda, ldw, ldc, dtype, 0, nullptr, 0, wstride, 0, batch, a_bstride, c_bstride, c_is_T, stream);
+  const int esz = dtype == 1 ? 2 : 4;
+  GemvArgs a{A, W, (float *)C, M, N, K, lda, ldw, ldc, 0, nullptr, wstride,
+             (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0 && (a_bstride * esz) % 16 == 0) ? 1 : 0,
+             nullptr, nullptr, 1, nullptr, 0.f, 0.f, batch > 0 ? batch : 0, a_bstride, c_bstride, c_is_T};
+  if (batch > 65535) return fail("mrs_hyb_gemm_batched: more than 65535 products in one batch");
+  dim3 grid((N + 3) / 4, 1, batch > 0 ? batch : 1);
+  hipStream_t s = (hipStream_t)stream;
+#define MRS_GEMVB(T) do { if (M <= 1) hipLaunchKernelGGL((gemv_rows_kernel<T, 1, IN_PLAIN>), grid, dim3(256), 0, s, a); else if (M <= 2) hipLaunchKernelGGL((gemv_rows_kernel<T, 2, IN_PLAIN>), grid, dim3(256), 0, s, a); \
+                          else if (M <= 4) hipLaunchKernelGGL((gemv_rows_kernel<T, 4, IN_PLAIN>), grid, dim3(256), 0, s, a); else hipLaunchKernelGGL((gemv_rows_kernel<T, 8, IN_PLAIN>), grid, dim3(256), 0, s, a); } while (0)
+  if (dtype == 1) MRS_GEMVB(mrs::bf16_t); else MRS_GEMVB(float);
+#undef MRS_GEMVB
+  return hipGetLastError() == hipSuccess ? 0 : fail("mrs_hyb_gemm_batched: launch failed");
 }
 
 /* in_mode: 0 plain (A in dtype), 1 GLU (A = f32 [M, 2 K] gate | up), 2 scaled rows (A = f32 source rows; row m = src_scale[r] * A[r / src_div], r = src_row[m]; no
@@ -444,7 +489,7 @@ extern "C" int mrs_hyb_gemv_act(const void *A, const void *W, float *C, int M, i
   const int esz = dtype == 1 ? 2 : 4;
   GemvArgs a{A, W, C, M, N, K, lda, ldw, ldc, accumulate, row_group, wstride,
              (K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && ((uintptr_t)A % 16) == 0 && ((uintptr_t)W % 16) == 0 && (wstride * esz) % 16 == 0 &&
-              (!in_bias || ((uintptr_t)in_bias % 16) == 0)) ? 1 : 0, src_row, src_scale, src_div, in_bias, p0, p1};
+              (!in_bias || ((uintptr_t)in_bias % 16) == 0)) ? 1 : 0, src_row, src_scale, src_div, in_bias, p0, p1, 0, 0, 0, 0};
   dim3 grid((N + 3) / 4, row_group ? M : 1);
   hipStream_t s = (hipStream_t)stream;
 #define MRS_GEMV_(T, MR, IN) hipLaunchKernelGGL((gemv_rows_kernel<T, MR, IN>), grid, dim3(256), 0, s, a)

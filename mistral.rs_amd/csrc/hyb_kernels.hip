@@ -42,64 +42,70 @@ template <class T> __global__ void __launch_bounds__(256) embed_kernel(const int
 }
 
 // ---------------------------------------------------------------------------------- x / sqrt(mean(x^2) + eps) * (w | 1 + w); grid.y = equal parts of the row
-// gate (optional, [rows, ldg]): the row is multiplied by silu(gate) BEFORE its root mean square is taken
+// w null: no weight.  gate (optional, [rows, ldg]): gate_after 0: the row is multiplied by silu(gate) BEFORE its root mean square is taken; gate_after 1: the normed row is
+// multiplied by silu(gate)
 template <class T> __global__ void __launch_bounds__(256) rmsnorm_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ w, T *__restrict__ out, float *__restrict__ out32,
-                                                                          float *__restrict__ rstd, int part, float eps, int one_plus, int ldo, const float *__restrict__ gate, int ldg) {
+                                                                          float *__restrict__ rstd, int part, float eps, int one_plus, int ldo, const float *__restrict__ gate, int ldg,
+                                                                          int gate_after) {
   __shared__ float red[4];
-  extern __shared__ float row[];  // the (gated) part, when a gate is given: silu is evaluated once
+  extern __shared__ float row[];  // the (gated) part, when a gate comes first: silu is evaluated once
   const int t = blockIdx.x, g = blockIdx.y;
   const float *xr = x + (size_t)t * ldx + (size_t)g * part;
   const float *gr = gate ? gate + (size_t)t * ldg + (size_t)g * part : nullptr;
+  const bool pre = gr && !gate_after;
   float s = 0.f;
   for (int c = threadIdx.x; c < part; c += 256) {
     float v = xr[c];
-    if (gr) { v *= silu_f(gr[c]); row[c] = v; }
+    if (pre) { v *= silu_f(gr[c]); row[c] = v; }
     s = fmaf(v, v, s);
   }
   s = block_sum_256(s, red);
   const float inv = 1.0f / sqrtf(s / (float)part + eps);
   if (rstd && threadIdx.x == 0) rstd[(size_t)t * gridDim.y + g] = inv;
   for (int c = threadIdx.x; c < part; c += 256) {
-    const float wv = w[(size_t)g * part + c];
-    const float v = (gr ? row[c] : xr[c]) * inv * (one_plus ? 1.0f + wv : wv);
+    const float wv = w ? w[(size_t)g * part + c] : (one_plus ? 0.f : 1.0f);
+    float v = (pre ? row[c] : xr[c]) * inv * (one_plus ? 1.0f + wv : wv);
+    if (gr && gate_after) v *= silu_f(gr[c]);
     if (out) out[(size_t)t * ldo + (size_t)g * part + c] = from_f<T>(v);
     if (out32) out32[(size_t)t * ldo + (size_t)g * part + c] = v;
   }
 }
 
-// ---------------------------------------------------------------------------------- short causal convolution + SiLU with carried taps
+// ---------------------------------------------------------------------------------- short causal convolution (+ SiLU) with carried taps
 // u [rows, ldu] (the channels start at column 0 of the pointer handed in), cw [C, taps] (the last column multiplies the current token), state [slots, C, taps - 1]
-// (oldest first).  An entry that starts at position 0 reads zeros instead of its slot.
-__global__ void __launch_bounds__(256) conv_silu_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ cw, const float *__restrict__ cb, const float *__restrict__ state,
-                                                        const int *__restrict__ tok_seq, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
-                                                        const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps) {
+// (oldest first).  An entry that starts at position 0 reads zeros instead of its slot.  in_bias (nullable, [C]): the bias of the product that made u -- the convolution
+// runs over u + in_bias, and that is what the slot carries.  cb (nullable): the convolution's own bias.  act 1: SiLU of the result, 0: the result as it is.
+__global__ void __launch_bounds__(256) conv_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw, const float *__restrict__ cb,
+                                                   const float *__restrict__ state, const int *__restrict__ tok_seq, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
+                                                   const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps, int act) {
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int s = tok_seq[t], r0 = seq_start[s], i = t - r0;
   const bool carried = seq_pos0[s] > 0;
   const float *st = state + ((size_t)seq_slot[s] * C + c) * (taps - 1);
-  float acc = cb[c];
+  const float ib = in_bias ? in_bias[c] : 0.f;
+  float acc = cb ? cb[c] : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int idx = i - (taps - 1) + j;
     float v = 0.f;
-    if (idx >= 0) v = u[(size_t)(r0 + idx) * ldu + c];
+    if (idx >= 0) v = u[(size_t)(r0 + idx) * ldu + c] + ib;
     else if (carried) v = st[(taps - 1) + idx];
     acc = fmaf(cw[(size_t)c * taps + j], v, acc);
   }
-  out[(size_t)t * C + c] = silu_f(acc);
+  out[(size_t)t * C + c] = act ? silu_f(acc) : acc;
 }
 // decode steps (every entry brings one row): convolution and tap shift in one launch, the thread of (entry, channel) reads its taps, then writes them
-__global__ void __launch_bounds__(256) conv_silu_step_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ cw, const float *__restrict__ cb, float *__restrict__ state,
-                                                             const int *__restrict__ seq_start, const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot,
-                                                             float *__restrict__ out, int C, int taps) {
+__global__ void __launch_bounds__(256) conv_step_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw, const float *__restrict__ cb,
+                                                        float *__restrict__ state, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot,
+                                                        float *__restrict__ out, int C, int taps, int act) {
   const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int row = seq_start[s], keep = taps - 1;
   if (seq_start[s + 1] - row != 1) return;
   const bool carried = seq_pos0[s] > 0;
   float *st = state + ((size_t)seq_slot[s] * C + c) * keep;
-  const float cur = u[(size_t)row * ldu + c];
-  float acc = cb[c], v[16];
+  const float cur = u[(size_t)row * ldu + c] + (in_bias ? in_bias[c] : 0.f);
+  float acc = cb ? cb[c] : 0.f, v[16];
 #pragma unroll
   for (int k = 0; k < 16; ++k) {
     if (k >= keep) break;
@@ -107,7 +113,7 @@ __global__ void __launch_bounds__(256) conv_silu_step_kernel(const float *__rest
     acc = fmaf(cw[(size_t)c * taps + k], v[k], acc);
   }
   acc = fmaf(cw[(size_t)c * taps + keep], cur, acc);
-  out[(size_t)row * C + c] = silu_f(acc);
+  out[(size_t)row * C + c] = act ? silu_f(acc) : acc;
 #pragma unroll
   for (int k = 0; k < 16; ++k) {
     if (k >= keep) break;
@@ -115,20 +121,21 @@ __global__ void __launch_bounds__(256) conv_silu_step_kernel(const float *__rest
   }
 }
 // the slot's taps after the step: the last taps - 1 inputs of (old taps ++ this step's rows).  One thread per (entry, channel) reads everything before it writes.
-__global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict__ u, int ldu, float *__restrict__ state, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
-                                                         const int *__restrict__ seq_slot, int C, int taps) {
+__global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, float *__restrict__ state, const int *__restrict__ seq_start,
+                                                         const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot, int C, int taps) {
   const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int r0 = seq_start[s], len = seq_start[s + 1] - r0, keep = taps - 1;
   if (len <= 0) return;
   const bool carried = seq_pos0[s] > 0;
   float *st = state + ((size_t)seq_slot[s] * C + c) * keep;
+  const float ib = in_bias ? in_bias[c] : 0.f;
   float v[16];
 #pragma unroll
   for (int k = 0; k < 16; ++k) {
     if (k >= keep) break;
     const int idx = len - keep + k;
-    v[k] = idx >= 0 ? u[(size_t)(r0 + idx) * ldu + c] : (carried ? st[keep + idx] : 0.f);
+    v[k] = idx >= 0 ? u[(size_t)(r0 + idx) * ldu + c] + ib : (carried ? st[keep + idx] : 0.f);
   }
 #pragma unroll
   for (int k = 0; k < 16; ++k) {
@@ -149,7 +156,8 @@ __global__ void __launch_bounds__(256) conv_state_kernel(const float *__restrict
 struct ScanArgs {
   const float *xbc;   // [rows, C]: x [heads * P] | B [G * N] | C [G * N] after convolution + SiLU
   const float *u;     // [rows, ldu] projection: dt_raw at column dt_col
-  const float *dt_bias, *A_log, *D;
+  const float *dt_bias, *A_log, *D;   // D nullable (no skip term)
+  const float *fixed_decay;  // [heads], nullable: every row steps with dt = 1 and this decay (dt_bias, A_log and the dt column of u are not read): S <- decay_h S + B x^T
   float *steps;       // [rows, heads, 2]: dt, decay
   float *state;       // [slots, heads, N, P]
   float *out;         // [rows, heads * P]
@@ -163,6 +171,11 @@ __global__ void __launch_bounds__(256) ssd_steps_kernel(ScanArgs a) {
   const int i = blockIdx.x * 256 + threadIdx.x;
   if (i >= a.rows * a.heads) return;
   const int t = i / a.heads, h = i % a.heads;
+  if (a.fixed_decay) {
+    a.steps[2 * (size_t)i] = 1.0f;
+    a.steps[2 * (size_t)i + 1] = a.fixed_decay[h];
+    return;
+  }
   const float dt = softplus_f(a.u[(size_t)t * a.ldu + a.dt_col + h] + a.dt_bias[h]);
   a.steps[2 * (size_t)i] = dt;
   a.steps[2 * (size_t)i + 1] = expf(-expf(a.A_log[h]) * dt);
@@ -202,7 +215,7 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
   float S[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) S[k] = (k < nk && init) ? init[(size_t)(r * K + k) * a.P + pc] : 0.f;
-  const float Dh = a.D[h];
+  const float Dh = a.D ? a.D[h] : 0.f;
   const int bcol = inner + g * a.N + r * K, ccol = inner + a.G * a.N + g * a.N + r * K;
   float B[DEPTH][K], Cv[DEPTH][K], prod = 1.0f;
   ScanStage sg[DEPTH];
@@ -232,8 +245,11 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
     g_.x = xr[h * a.P + pc];
     float d0, d1;
     if (DEPTH == 1 && !LOCAL) {  // decode steps: the step size and decay inline (ssd_steps_kernel's expressions), one launch less
-      d0 = softplus_f(a.u[(size_t)row * a.ldu + a.dt_col + h] + a.dt_bias[h]);
-      d1 = expf(-expf(a.A_log[h]) * d0);
+      if (a.fixed_decay) { d0 = 1.0f; d1 = a.fixed_decay[h]; }
+      else {
+        d0 = softplus_f(a.u[(size_t)row * a.ldu + a.dt_col + h] + a.dt_bias[h]);
+        d1 = expf(-expf(a.A_log[h]) * d0);
+      }
     } else {
       const float *de = a.steps + 2 * ((size_t)row * a.heads + h);
       d0 = de[0]; d1 = de[1];
@@ -296,7 +312,7 @@ template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_b
   float S[K];
 #pragma unroll
   for (int k = 0; k < K; ++k) S[k] = (k < nk && init) ? init[(size_t)(r * K + k) * P + pc] : 0.f;
-  const float Dh = a.D[h];
+  const float Dh = a.D ? a.D[h] : 0.f;
   const int bcol = inner + g * N, ccol = inner + a.G * N + g * N, per = TC * rowpad, rowlen = 2 * N + P + 2;
   float stg[16], prod = 1.0f;
   auto fetch = [&](int c0) {
@@ -442,7 +458,8 @@ template <class T> __global__ void __launch_bounds__(256) qk_norm_rope_cache_ker
 
 // ---------------------------------------------------------------------------------- paged attention, sliding window with kept first tokens
 // Query at position i sees key j <= i when i - j < window or j < keep_first (window <= 0: every j <= i).  One wave per (row, head): keys in passes of 64 (a lane = a key for the
-// scores, a lane = value dimensions for the weighted sum), running maximum / sum in f32.
+// scores, a lane = value dimensions for the weighted sum), running maximum / sum in f32.  Options: softcap > 0: s <- softcap tanh(s / softcap) after the scale; sink: one
+// more term e^0 in the softmax's denominator (a key of score 0 without a value); gate (f32 [rows, ldg], column head * Dv + d): the output is multiplied by sigmoid(gate).
 struct AttnArgs {
   const void *q;        // [rows, H * D] in T
   const void *k_cache, *v_cache;
@@ -451,7 +468,12 @@ struct AttnArgs {
   void *out;            // [rows, H * Dv] in T
   int H, G, D, Dv, block_size, max_blocks, window, keep_first;
   float scale;
+  float softcap;        // 0: none
+  int sink;
+  const float *gate;    // nullable
+  int ldg;
 };
+__device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 template <class T> struct Ld;
 template <> struct Ld<bf16_t> {
   static __device__ __forceinline__ void v8(const bf16_t *p, float *o) {
@@ -488,7 +510,7 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
   int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;  // kept first tokens that the window does not already cover
   if (n1 < 0) n1 = 0;
   const int total = n1 + (i - w_lo + 1);
-  float m = -FLT_MAX, l = 0.f, o[DVC][2];
+  float m = a.sink ? 0.f : -FLT_MAX, l = a.sink ? 1.f : 0.f, o[DVC][2];
 #pragma unroll
   for (int c = 0; c < DVC; ++c) o[c][0] = o[c][1] = 0.f;
   MRS_WAVE_SYNC();
@@ -512,7 +534,7 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
       } else {
         for (int d = 0; d < a.D; ++d) acc = fmaf(qs[d], to_f<T>(kr[d]), acc);
       }
-      sc = acc * a.scale;
+      sc = capped(acc * a.scale, a.softcap);
     }
     const float mn = fmaxf(m, wave_max(sc));
     const float alpha = expf(m - mn);
@@ -552,11 +574,12 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
   }
   const float inv = 1.0f / l;
   T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
+  const float *gr = a.gate ? a.gate + (size_t)t * a.ldg + (size_t)h * a.Dv : nullptr;
 #pragma unroll
   for (int c = 0; c < DVC; ++c) {
     const int d = 128 * c + 2 * lane;
-    if (d < a.Dv) out[d] = from_f<T>(o[c][0] * inv);
-    if (d + 1 < a.Dv) out[d + 1] = from_f<T>(o[c][1] * inv);
+    if (d < a.Dv) out[d] = from_f<T>(o[c][0] * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
+    if (d + 1 < a.Dv) out[d + 1] = from_f<T>(o[c][1] * inv * (gr ? sigmoid_f(gr[d + 1]) : 1.0f));
   }
 }
 
@@ -588,7 +611,7 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
   float m[NQ], l[NQ], o[NQ][DVC][2];
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
-    m[q] = -FLT_MAX; l[q] = 0.f;
+    m[q] = a.sink ? 0.f : -FLT_MAX; l[q] = a.sink ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < DVC; ++c) o[q][c][0] = o[q][c][1] = 0.f;
   }
@@ -622,7 +645,7 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
     for (int q = 0; q < NQ; ++q) {
       const int iq = i0 + q;
       const bool vis = key >= 0 && q < nq && key <= iq && (a.window <= 0 || iq - key < a.window || key < a.keep_first);
-      const float sv = vis ? sc[q] * a.scale : -FLT_MAX;
+      const float sv = vis ? capped(sc[q] * a.scale, a.softcap) : -FLT_MAX;
       const float mn = fmaxf(m[q], wave_max(sv));
       const float alpha = expf(m[q] - mn);
       const float pq = vis ? expf(sv - mn) : 0.f;
@@ -664,10 +687,14 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
     if (q >= nq) break;
     const float inv = 1.0f / l[q];
     T *out = (T *)a.out + ((size_t)(t0 + q) * a.H + h) * a.Dv;
+    const float *gr = a.gate ? a.gate + (size_t)(t0 + q) * a.ldg + (size_t)h * a.Dv : nullptr;
 #pragma unroll
     for (int c = 0; c < DVC; ++c) {
       const int d = 128 * c + 2 * lane;
-      if (d < a.Dv) { out[d] = from_f<T>(o[q][c][0] * inv); out[d + 1] = from_f<T>(o[q][c][1] * inv); }
+      if (d < a.Dv) {
+        out[d] = from_f<T>(o[q][c][0] * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
+        out[d + 1] = from_f<T>(o[q][c][1] * inv * (gr ? sigmoid_f(gr[d + 1]) : 1.0f));
+      }
     }
   }
 }
@@ -908,6 +935,102 @@ template <class T> __global__ void __launch_bounds__(256) qkv_bias_temp_cache_ke
     ((T *)a.v_cache)[(((size_t)blk * a.G + g) * a.block_size + off) * a.Dv + d] = from_f<T>(v[e] + (a.vb ? a.vb[e] : 0.f));
   }
 }
+// ---------------------------------------------------------------------------------- half-split rotary on f32 rows, in place (queries and keys of a recurrence)
+// u [rows, ld]: `heads` heads of D values from column col.  In the first `rot` dimensions of a head, (x_i, x_{i + rot / 2}) turns by position * freq[i]; then every value of
+// the head is multiplied by mult.  grid.y = 0: the range at q_col (mult 1), 1: the range at k_col (mult k_mult).
+__global__ void __launch_bounds__(256) rotary_half_kernel(float *__restrict__ u, int ld, int q_col, int k_col, int heads, int D, int rot, const float *__restrict__ freq,
+                                                          const int *__restrict__ tok_pos, float k_mult) {
+  const int t = blockIdx.x, half = rot >> 1;
+  float *row = u + (size_t)t * ld + (blockIdx.y ? k_col : q_col);
+  const float mult = blockIdx.y ? k_mult : 1.0f, pos = (float)tok_pos[t];
+  const int per = D - half;  // items of a head: `half` pairs, then the D - rot values that pass
+  for (int e = threadIdx.x; e < heads * per; e += 256) {
+    const int h = e / per, i = e - h * per;
+    float *x = row + (size_t)h * D;
+    if (i < half) {
+      float sn, cs;
+      sincosf(pos * freq[i], &sn, &cs);
+      const float a = x[i], b = x[i + half];
+      x[i] = (a * cs - b * sn) * mult;
+      x[i + half] = (b * cs + a * sn) * mult;
+    } else {
+      x[i + half] *= mult;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------- latent attention: the query rounded, the latent row normed and paged
+// u [rows, ld] = q [nq] | c [R] (f32, one product): q goes to q_out (T) as it is; c / rms(c) * w (plain weight) goes to the row's page slot of c_cache [blocks, 1, block_size, R]
+template <class T> __global__ void __launch_bounds__(256) latent_norm_cache_kernel(const float *__restrict__ u, int ld, int nq, int R, const float *__restrict__ w,
+                                                                                   const long long *__restrict__ slot_mapping, T *__restrict__ q_out, T *__restrict__ c_cache, float eps) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float *q = u + (size_t)t * ld, *c = q + nq;
+  for (int e = tid; e < nq; e += 256) q_out[(size_t)t * nq + e] = from_f<T>(q[e]);
+  float s = 0.f;
+  for (int e = tid; e < R; e += 256) s = fmaf(c[e], c[e], s);
+  const float inv = 1.0f / sqrtf(block_sum_256(s, red) / (float)R + eps);
+  const long long slot = slot_mapping[t];
+  if (slot < 0) return;
+  for (int e = tid; e < R; e += 256) c_cache[(size_t)slot * R + e] = from_f<T>(c[e] * inv * w[e]);
+}
+
+// ---------------------------------------------------------------------------------- several residual streams (hyper-connections)
+// x [rows, S, W] f32.  One launch closes a sublayer and opens the next:
+//   write  (y given): new_r = sum_s mix[s, r] x_s + outw[r] y for every stream r, all from the old streams (mix null: new_r = outw[r] y -- the streams' start)
+//   read   (inw given): v = sum_s inw[s] x_s of the updated streams; norm_w given: v / rms(v) * (1 + norm_w | norm_w) to out (T) and / or out32; norm_w null: v itself to out32
+template <class T, int S> __global__ void __launch_bounds__(256) hyper_step_kernel(float *__restrict__ x, const float *__restrict__ y, const float *__restrict__ mix,
+                                                                                   const float *__restrict__ outw, const float *__restrict__ inw, const float *__restrict__ norm_w,
+                                                                                   T *__restrict__ out, float *__restrict__ out32, int W, float eps, int one_plus) {
+  __shared__ float red[4];
+  __shared__ float cm[S * S], co[S], ci[S];
+  extern __shared__ float row[];  // the read sum, until its norm is known
+  const int t = blockIdx.x, tid = threadIdx.x;
+  if (tid < S * S) cm[tid] = mix ? mix[tid] : 0.f;
+  if (tid < S) { co[tid] = outw ? outw[tid] : 0.f; ci[tid] = inw ? inw[tid] : 0.f; }
+  __syncthreads();
+  float *xr = x + (size_t)t * S * W;
+  float ss = 0.f;
+  for (int c = tid; c < W; c += 256) {
+    float v[S];
+    if (y) {
+      const float yv = y[(size_t)t * W + c];
+      float old[S];
+      if (mix) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) old[s] = xr[(size_t)s * W + c];
+      }
+#pragma unroll
+      for (int r = 0; r < S; ++r) {
+        float acc = 0.f;
+        if (mix) {
+#pragma unroll
+          for (int s = 0; s < S; ++s) acc = fmaf(cm[s * S + r], old[s], acc);
+        }
+        v[r] = fmaf(co[r], yv, acc);
+        xr[(size_t)r * W + c] = v[r];
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < S; ++s) v[s] = xr[(size_t)s * W + c];
+    }
+    if (inw) {
+      float uv = 0.f;
+#pragma unroll
+      for (int s = 0; s < S; ++s) uv = fmaf(ci[s], v[s], uv);
+      if (norm_w) { row[c] = uv; ss = fmaf(uv, uv, ss); }
+      else if (out32) out32[(size_t)t * W + c] = uv;
+    }
+  }
+  if (!inw || !norm_w) return;
+  const float inv = 1.0f / sqrtf(block_sum_256(ss, red) / (float)W + eps);
+  for (int c = tid; c < W; c += 256) {
+    const float v = row[c] * inv * (one_plus ? 1.0f + norm_w[c] : norm_w[c]);
+    if (out) out[(size_t)t * W + c] = from_f<T>(v);
+    if (out32) out32[(size_t)t * W + c] = v;
+  }
+}
+
 __global__ void __launch_bounds__(256) gather_rows_kernel(const float *__restrict__ x, const int *__restrict__ idx, float *__restrict__ out, int W) {
   const int i = blockIdx.x;
   for (int c = threadIdx.x; c < W; c += 256) out[(size_t)i * W + c] = x[(size_t)idx[i] * W + c];
@@ -931,42 +1054,47 @@ extern "C" int mrs_hyb_embed(const int *tokens, const void *table, float *x, int
 
 // parts > 1: every row is normed in `parts` equal pieces, each by its own root mean square.  out (dtype) and / or out32 (f32) receive the result, rstd [rows, parts] the 1 / rms.
 extern "C" int mrs_hyb_rmsnorm(const float *x, int ldx, const float *w, void *out, float *out32, float *rstd, int rows, int width, int parts, float eps, int one_plus, int dtype,
-                               const float *gate, int ldg, void *stream) {
+                               const float *gate, int ldg, int gate_after, void *stream) {
   if (rows <= 0) return 0;
   if (parts <= 0 || width % parts) return fail("mrs_hyb_rmsnorm: the row does not split into equal parts");
   dim3 grid(rows, parts);
-  const size_t lds = gate ? (size_t)(width / parts) * 4 : 0;
+  const size_t lds = gate && !gate_after ? (size_t)(width / parts) * 4 : 0;
   if (lds > 60000) return fail("mrs_hyb_rmsnorm: a gated part above 15000 values");
-  if (dtype == 1) hipLaunchKernelGGL(rmsnorm_kernel<mrs::bf16_t>, grid, dim3(256), lds, S_(stream), x, ldx, w, (mrs::bf16_t *)out, out32, rstd, width / parts, eps, one_plus, width, gate, ldg);
-  else if (dtype == 2) hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, dim3(256), lds, S_(stream), x, ldx, w, (float *)out, out32, rstd, width / parts, eps, one_plus, width, gate, ldg);
+  if (dtype == 1) hipLaunchKernelGGL(rmsnorm_kernel<mrs::bf16_t>, grid, dim3(256), lds, S_(stream), x, ldx, w, (mrs::bf16_t *)out, out32, rstd, width / parts, eps, one_plus, width, gate, ldg, gate_after);
+  else if (dtype == 2) hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, dim3(256), lds, S_(stream), x, ldx, w, (float *)out, out32, rstd, width / parts, eps, one_plus, width, gate, ldg, gate_after);
   else return fail("mrs_hyb_rmsnorm: dtype");
   return ok_or("mrs_hyb_rmsnorm");
 }
 
+/* out [rows, C] = act(conv(u + in_bias) + cb): in_bias, cb nullable; act 1 = SiLU, 0 = none.  The slots carry the last taps - 1 rows of u + in_bias. */
+extern "C" int mrs_hyb_conv(const float *u, int ldu, const float *in_bias, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start,
+                            const int *seq_pos0, const int *seq_slot, float *out, int rows, int entries, int C, int taps, int act, void *stream) {
+  if (rows <= 0) return 0;
+  if (taps < 1 || taps > 17) return fail("mrs_hyb_conv: 1 .. 17 taps");
+  if (rows == entries) {  // one row per entry (an entry without rows cannot occur then)
+    hipLaunchKernelGGL(conv_step_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, seq_start, seq_pos0, seq_slot, out, C, taps, act);
+    return ok_or("mrs_hyb_conv");
+  }
+  hipLaunchKernelGGL(conv_kernel, dim3(rows, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps, act);
+  if (taps > 1)
+    hipLaunchKernelGGL(conv_state_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, in_bias, state, seq_start, seq_pos0, seq_slot, C, taps);
+  return ok_or("mrs_hyb_conv");
+}
 extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start, const int *seq_pos0,
                                  const int *seq_slot, float *out, int rows, int entries, int C, int taps, void *stream) {
-  if (rows <= 0) return 0;
-  if (taps < 1 || taps > 17) return fail("mrs_hyb_conv_silu: 1 .. 17 taps");
-  if (rows == entries) {  // one row per entry (an entry without rows cannot occur then)
-    hipLaunchKernelGGL(conv_silu_step_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, cw, cb, state, seq_start, seq_pos0, seq_slot, out, C, taps);
-    return ok_or("mrs_hyb_conv_silu");
-  }
-  hipLaunchKernelGGL(conv_silu_kernel, dim3(rows, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps);
-  if (taps > 1)
-    hipLaunchKernelGGL(conv_state_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, state, seq_start, seq_pos0, seq_slot, C, taps);
-  return ok_or("mrs_hyb_conv_silu");
+  return mrs_hyb_conv(u, ldu, nullptr, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, rows, entries, C, taps, 1, stream);
 }
 
 /* steps: scratch [rows, heads, 2] f32.  Segment table (host-built): seg_entry / seg_row0 / seg_len [segments], ent_seg0 [entries + 1]; carry [segments, heads, N, P] and
  * decay [segments, heads] are scratch that is only touched when some entry has more than one segment (segments > entries). */
-extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, float *state, float *out, const int *seq_pos0,
-                                const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry,
-                                float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
+static int scan_launch(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, const float *fixed_decay, float *state, float *out,
+                       const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry,
+                       float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
   if (entries <= 0 || rows <= 0 || segments <= 0) return 0;
   if (heads <= 0 || G <= 0 || heads % G || P <= 0 || N <= 0) return fail("mrs_hyb_ssd_scan: bad head / group sizes");
   if (segments > 65535 || entries > 65535) return fail("mrs_hyb_ssd_scan: more than 65535 segments in one step");
   if (segments > entries && (!carry || !decay)) return fail("mrs_hyb_ssd_scan: segmented entries need the carry scratch");
-  ScanArgs a{xbc, u, dt_bias, A_log, D, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows};
+  ScanArgs a{xbc, u, dt_bias, A_log, D, fixed_decay, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows};
   const bool vec = C % 4 == 0 && (heads * P) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
   const bool single = rows == segments;  // one row per segment (decode steps): no ring, step sizes inline
   if (!single) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
@@ -1002,6 +1130,24 @@ extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *d
   return ok_or("mrs_hyb_ssd_scan");
 }
 
+extern "C" int mrs_hyb_ssd_scan(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, float *state, float *out, const int *seq_pos0,
+                                const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry,
+                                float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
+  if (!dt_bias || !A_log || !D || !u) return fail("mrs_hyb_ssd_scan: step-size bias, decay rate and skip weight are needed");
+  return scan_launch(xbc, u, dt_bias, A_log, D, nullptr, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, steps, carry, decay, rows, entries, segments, C, ldu,
+                     dt_col, heads, P, N, G, stream);
+}
+/* The same recurrence with one fixed decay per head and unit steps, S <- decay_h S + k v^T, o = S^T q (retention / decayed linear attention): xkq [rows, ld] holds
+ * v [heads * P] | k [G * N] | q [G * N] from column 0; state [slots, heads, N, P] */
+extern "C" int mrs_hyb_decay_scan(const float *xkq, int ld, const float *fixed_decay, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry,
+                                  const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry, float *decay, int rows, int entries, int segments,
+                                  int heads, int P, int N, int G, void *stream) {
+  if (!fixed_decay) return fail("mrs_hyb_decay_scan: the heads' decays are needed");
+  if (ld < heads * P + 2 * G * N) return fail("mrs_hyb_decay_scan: rows shorter than v | k | q");
+  return scan_launch(xkq, nullptr, nullptr, nullptr, nullptr, fixed_decay, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, steps, carry, decay, rows,
+                     entries, segments, ld, 0, 0, heads, P, N, G, stream);
+}
+
 extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping,
                                           void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype,
                                           void *stream) {
@@ -1016,12 +1162,13 @@ extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float 
 
 /* seg_entry / seg_row0 / seg_len [segments] (nullable): the batch's segment table (rows of one entry in pieces); with it, batches that bring portions run the
  * query-tiled kernel */
-extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
-                                         int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
-                                         const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream) {
+static int attn_launch(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
+                       int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
+                       const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg, void *stream) {
   if (rows <= 0) return 0;
-  if (Dv > 256 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 256 / heads % kv_heads");
-  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale};
+  if (Dv > 512 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 512 / heads % kv_heads");
+  if (gate && ldg < H * Dv) return fail("mrs_hyb_paged_window_attn: gate rows shorter than heads * value size");
+  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg};
   const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
   const int c = (Dv + 127) / 128;
   if (vec && seg_entry && segments > 0 && rows > segments && segments <= 65535 && seg_rows > 0) {
@@ -1030,8 +1177,8 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
     if (lds <= 65536) {
       dim3 grid((seg_rows + NQ - 1) / NQ, H, segments);
 #define MRS_ATTN_T(T, C) hipLaunchKernelGGL((paged_window_attn_tile_kernel<T, C, NQ>), grid, dim3(64), lds, S_(stream), a, seg_entry, seg_row0, seg_len)
-      if (dtype == 1) { if (c <= 1) MRS_ATTN_T(mrs::bf16_t, 1); else MRS_ATTN_T(mrs::bf16_t, 2); }
-      else if (dtype == 2) { if (c <= 1) MRS_ATTN_T(float, 1); else MRS_ATTN_T(float, 2); }
+      if (dtype == 1) { if (c <= 1) MRS_ATTN_T(mrs::bf16_t, 1); else if (c <= 2) MRS_ATTN_T(mrs::bf16_t, 2); else MRS_ATTN_T(mrs::bf16_t, 4); }
+      else if (dtype == 2) { if (c <= 1) MRS_ATTN_T(float, 1); else if (c <= 2) MRS_ATTN_T(float, 2); else MRS_ATTN_T(float, 4); }
       else return fail("mrs_hyb_paged_window_attn: dtype");
 #undef MRS_ATTN_T
       return ok_or("mrs_hyb_paged_window_attn");
@@ -1041,11 +1188,26 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
   dim3 grid(rows, H);
 #define MRS_ATTN(T, C) do { if (vec) hipLaunchKernelGGL((paged_window_attn_kernel<T, C, true>), grid, dim3(64), lds, S_(stream), a); \
                             else hipLaunchKernelGGL((paged_window_attn_kernel<T, C, false>), grid, dim3(64), lds, S_(stream), a); } while (0)
-  if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else MRS_ATTN(mrs::bf16_t, 2); }
-  else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else MRS_ATTN(float, 2); }
+  if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else if (c <= 2) MRS_ATTN(mrs::bf16_t, 2); else MRS_ATTN(mrs::bf16_t, 4); }
+  else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else if (c <= 2) MRS_ATTN(float, 2); else MRS_ATTN(float, 4); }
   else return fail("mrs_hyb_paged_window_attn: dtype");
 #undef MRS_ATTN
   return ok_or("mrs_hyb_paged_window_attn");
+}
+
+extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
+                                         int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
+                                         const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream) {
+  return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, dtype, seg_entry, seg_row0, seg_len,
+                     segments, seg_rows, 0.f, 0, nullptr, 0, stream);
+}
+/* the same attention with its options: softcap (0: none), sink (a zero-score term in the denominator), gate (nullable f32 [rows, ldg]: output times sigmoid(gate)) */
+extern "C" int mrs_hyb_paged_attn_opts(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
+                                       int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
+                                       const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg,
+                                       void *stream) {
+  return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, dtype, seg_entry, seg_row0, seg_len,
+                     segments, seg_rows, softcap, sink, gate, ldg, stream);
 }
 
 /* h [rows, W] f32 (contiguous), wr [E (+ 1), W] f32 */
@@ -1166,4 +1328,50 @@ extern "C" int mrs_hyb_gather_rows(const float *x, const int *idx, float *out, i
   if (n <= 0) return 0;
   hipLaunchKernelGGL(gather_rows_kernel, dim3(n), dim3(256), 0, S_(stream), x, idx, out, W);
   return ok_or("mrs_hyb_gather_rows");
+}
+
+/* In place on u [rows, ld]: heads x D values at q_col and at k_col; the first rot dimensions of every head turn in half-split pairs (i, i + rot / 2) by tok_pos * freq[i];
+ * the key range is then multiplied by k_mult.  k_col < 0: queries only. */
+extern "C" int mrs_hyb_rotary_half(float *u, int ld, int q_col, int k_col, int heads, int D, int rot, const float *freq, const int *tok_pos, float k_mult, int rows, void *stream) {
+  if (rows <= 0) return 0;
+  if (heads <= 0 || D <= 0 || rot < 0 || (rot & 1) || rot > D || (rot > 0 && !freq)) return fail("mrs_hyb_rotary_half: even rot <= dim");
+  hipLaunchKernelGGL(rotary_half_kernel, dim3(rows, k_col >= 0 ? 2 : 1), dim3(256), 0, S_(stream), u, ld, q_col, k_col, heads, D, rot, freq, tok_pos, k_mult);
+  return ok_or("mrs_hyb_rotary_half");
+}
+
+/* u [rows, ld] = q [nq] | c [R]: q_out [rows, nq] (dtype) = q; c_cache[slot] (dtype, rows of R) = c / rms(c) * w */
+extern "C" int mrs_hyb_latent_norm_cache(const float *u, int ld, int nq, int R, const float *w, const long long *slot_mapping, void *q_out, void *c_cache, float eps, int rows, int dtype,
+                                         void *stream) {
+  if (rows <= 0) return 0;
+  if (nq <= 0 || R <= 0 || ld < nq + R || !w) return fail("mrs_hyb_latent_norm_cache: rows shorter than q | latent, or no norm weight");
+  if (dtype == 1) hipLaunchKernelGGL(latent_norm_cache_kernel<mrs::bf16_t>, dim3(rows), dim3(256), 0, S_(stream), u, ld, nq, R, w, slot_mapping, (mrs::bf16_t *)q_out, (mrs::bf16_t *)c_cache, eps);
+  else if (dtype == 2) hipLaunchKernelGGL(latent_norm_cache_kernel<float>, dim3(rows), dim3(256), 0, S_(stream), u, ld, nq, R, w, slot_mapping, (float *)q_out, (float *)c_cache, eps);
+  else return fail("mrs_hyb_latent_norm_cache: dtype");
+  return ok_or("mrs_hyb_latent_norm_cache");
+}
+
+/* x [rows, S, W] f32 residual streams.  y (nullable, [rows, W]): x_r <- sum_s mix[s, r] x_s + outw[r] y (mix null: x_r <- outw[r] y).  inw (nullable, [S]): v = sum_s inw[s] x_s of
+ * the updated streams; with norm_w the RMS-normed v goes to out (dtype, nullable) / out32 (nullable), without it v goes to out32. */
+extern "C" int mrs_hyb_hyper_step(float *x, const float *y, const float *mix, const float *outw, const float *inw, const float *norm_w, void *out, float *out32, int rows, int S, int W,
+                                  float eps, int one_plus, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (S < 1 || S > 8) return fail("mrs_hyb_hyper_step: 1 .. 8 streams");
+  if (W <= 0 || W > 15000) return fail("mrs_hyb_hyper_step: 1 .. 15000 values per row");
+  if (y && !outw) return fail("mrs_hyb_hyper_step: writing needs the streams' output weights");
+  if (dtype != 1 && dtype != 2) return fail("mrs_hyb_hyper_step: dtype");
+  const size_t lds = inw && norm_w ? (size_t)W * 4 : 0;
+#define MRS_HC(S_N) do { if (dtype == 1) hipLaunchKernelGGL((hyper_step_kernel<mrs::bf16_t, S_N>), dim3(rows), dim3(256), lds, S_(stream), x, y, mix, outw, inw, norm_w, (mrs::bf16_t *)out, out32, W, eps, one_plus); \
+                         else hipLaunchKernelGGL((hyper_step_kernel<float, S_N>), dim3(rows), dim3(256), lds, S_(stream), x, y, mix, outw, inw, norm_w, (float *)out, out32, W, eps, one_plus); } while (0)
+  switch (S) {
+    case 1: MRS_HC(1); break;
+    case 2: MRS_HC(2); break;
+    case 3: MRS_HC(3); break;
+    case 4: MRS_HC(4); break;
+    case 5: MRS_HC(5); break;
+    case 6: MRS_HC(6); break;
+    case 7: MRS_HC(7); break;
+    default: MRS_HC(8); break;
+  }
+#undef MRS_HC
+  return ok_or("mrs_hyb_hyper_step");
 }

@@ -32,7 +32,14 @@ DTYPES = {"bfloat16": (1, torch.bfloat16), "float32": (2, torch.float32)}
 
 _SIGS = {
     "mrs_hyb_embed": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "mrs_hyb_rmsnorm": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _i, _vp],
+    "mrs_hyb_rmsnorm": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _i, _i, _vp],
+    "mrs_hyb_conv": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "mrs_hyb_decay_scan": [_vp, _i] + [_vp] * 12 + [_i] * 7 + [_vp],
+    "mrs_hyb_paged_attn_opts": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _i, _vp],
+    "mrs_hyb_rotary_half": [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _f, _i, _vp],
+    "mrs_hyb_latent_norm_cache": [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _i, _vp],
+    "mrs_hyb_hyper_step": [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _vp],
+    "mrs_hyb_gemm_batched": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _l, _l, _l, _i, _vp],
     "mrs_hyb_conv_silu": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "mrs_hyb_ssd_scan": [_vp] * 16 + [_i] * 10 + [_vp],
     "mrs_hyb_qk_norm_rope_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
@@ -154,11 +161,13 @@ class RaggedBatch:
 # ------------------------------------------------------------------------------------------------------------------ layer descriptions
 @dataclass
 class RotarySpec:
-    """Interleaved rotary on the first `dims` dimensions of a head: pair (2i, 2i + 1) turns by position * f_i, f_i = base^(-2i / dims), optionally rescaled by wavelength
-    (`scaling`: factor, low, high, original -- wavelengths under original / high keep f, over original / low use f / factor, linear blend between)."""
+    """Rotary on the first `dims` dimensions of a head: a pair turns by position * f_i, f_i = base^(-2i / dims), optionally rescaled by wavelength (`scaling`: factor, low,
+    high, original -- wavelengths under original / high keep f, over original / low use f / factor, linear blend between).  `layout`: "interleaved" pairs (2i, 2i + 1) or
+    "half" pairs (i, i + dims / 2)."""
     dims: int
     base: float
     scaling: Optional[dict] = None
+    layout: str = "interleaved"
 
     def frequencies(self) -> np.ndarray:
         i = np.arange(self.dims // 2, dtype=np.float64)
@@ -197,6 +206,42 @@ class TalkAttentionSpec:
     temp_coef: float = 0.0     # query factor 1 + temp_coef ln(floor((pos + 1) / temp_every) + 1); temp_every 0: none
     temp_every: int = 0
     kv_from: Optional[int] = None   # index of the layer whose K / V pages this layer reads (it has no key / value projections then)
+
+
+@dataclass
+class SinkAttentionSpec:
+    """Causal softmax attention with a zero-score sink, capped scores, convolved projections, a query temperature and an elementwise output gate (GatedSinkAttention)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    conv: int = 0              # taps of the causal convolution over q / k / v (0: none)
+    softcap: float = 0.0       # 0: scores are not capped
+    temp_coef: float = 0.0     # query factor 1 + temp_coef ln(floor((pos + 1) / temp_every) + 1); temp_every 0: none
+    temp_every: int = 0
+    kv_from: Optional[int] = None   # index of the layer whose K / V pages this layer reads (it has no key / value projections then)
+    sink: bool = True
+
+
+@dataclass
+class RetentionSpec:
+    """Decayed linear attention: per head S <- decay S + k v^T, o = S^T q (RetentionMixer)."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: List[float]
+    rotary: Optional[RotarySpec] = None
+
+
+@dataclass
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are expanded from one cached low-rank row per token (LatentAttention)."""
+    heads: int
+    dim: int
+    vdim: int
+    kv_rank: int
+    scale: float
 
 
 @dataclass
@@ -247,6 +292,13 @@ class DenseSpec:
 
 
 @dataclass
+class GluSpec:
+    """down(silu(gate h) * (up h)) (GluFeedForward)."""
+    ff: int
+    kind = "dense_glu_silu"
+
+
+@dataclass
 class LayerSpec:
     kind: str
     mixer: object
@@ -265,6 +317,9 @@ class HybridSpec:
     head: str = "head"
     norm: str = "rms_one_plus"   # "rms_one_plus": x / rms * (1 + w);  "layer": (x - mean) / sqrt(var + eps) * w + b, the bias being the tensor `<name>.b`
     post_norms: bool = False     # every sublayer's output is normed (`norm1b` / `norm2b`) before it joins the residual stream
+    embed_norm: Optional[str] = None   # tensor of a norm (of the model's kind) applied to the embedding rows
+    residual_mult: float = 1.0   # every sublayer's output is multiplied by this before it joins the residual stream(s)
+    streams: int = 0             # > 0: that many residual streams with per-sublayer read / write / mixing weights (`hc1.*` / `hc2.*`: in [S], out [S], mix [S, S] from -> to)
 
 
 def gekilix_spec(cfg: dict) -> HybridSpec:
@@ -328,9 +383,54 @@ def sobunex_spec(cfg: dict) -> HybridSpec:
     return HybridSpec(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, norm="layer", post_norms=True)
 
 
+def setopel_spec(cfg: dict) -> HybridSpec:
+    """config.json of a Setopel checkpoint -> the layer list: a normed embedding, one-plus RMS norms in front of every sublayer, sublayer outputs scaled by `residual_mult`,
+    optionally several residual streams; mixers `attention` (sink softmax, convolved q / k / v, some reading an earlier layer's pages), `retention` and `latent_attention`;
+    SiLU-GLU feed-forwards.  Every size and every model-dependent constant comes from the file; a key that is absent switches its mechanism off."""
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind == "attention":
+            qt = m.get("q_temp") or {}
+            src = m.get("kv_from")
+            if src is not None and not 0 <= int(src) < i:
+                raise ValueError(f"Setopel: layer {i} reads the keys of layer {src}, which does not run before it")
+            mixer = SinkAttentionSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m["vdim"]), float(m["scale"]), int(m.get("conv", 0) or 0),
+                                      float(m.get("softcap", 0.0) or 0.0), float(qt.get("coef", 0.0) or 0.0), int(qt.get("every", 0) or 0) if qt.get("coef") else 0,
+                                      None if src is None else int(src))
+            kind = "sink_attention"
+        elif kind == "retention":
+            rot = m.get("rot")
+            decay = [float(d) for d in m["decay"]]
+            if len(decay) != int(m["heads"]):
+                raise ValueError(f"Setopel: layer {i} lists {len(decay)} decays for {m['heads']} heads")
+            mixer = RetentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), decay,
+                                  RotarySpec(int(rot["dims"]), float(rot["base"]), None, "half") if rot and int(rot.get("dims", 0)) > 0 else None)
+        elif kind == "latent_attention":
+            mixer = LatentAttentionSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), int(m["kv_rank"]), float(m["scale"]))
+        else:
+            raise ValueError(f"Setopel: unknown layer type {L['type']!r}")
+        f = L.get("mlp")
+        ff = None
+        if f:
+            if f.get("kind") != "dense":
+                raise ValueError(f"Setopel: unknown feed-forward kind {f.get('kind')!r}")
+            ff = GluSpec(int(f["ff"]))
+        layers.append(LayerSpec(kind, mixer, ff, f"l{i}."))
+    for i, ls in enumerate(layers):
+        j = getattr(ls.mixer, "kv_from", None)
+        if j is not None:
+            o = layers[j].mixer
+            if not isinstance(o, SinkAttentionSpec) or o.kv_from is not None or (o.kv_heads, o.dim, o.vdim) != (ls.mixer.kv_heads, ls.mixer.dim, ls.mixer.vdim):
+                raise ValueError(f"Setopel: layer {i} cannot read the keys and values of layer {j} (no projections of its own there, or other head sizes)")
+    return HybridSpec(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, embed_norm="embed.norm", residual_mult=float(cfg.get("residual_mult", 1.0)),
+                      streams=int(cfg.get("streams", 0) or 0))
+
+
 # ------------------------------------------------------------------------------------------------------------------ mixers and feed-forwards
 class _Module:
     out_bias = None            # f32 bias of the module's last product, left to the caller (a norm that follows adds it while it reads the product)
+    wants_f32_input = False    # feed-forwards: the normed rows are needed in f32 too (routers)
 
     def __init__(self, model: "HybridDecoder"):
         self.m = model
@@ -499,6 +599,8 @@ class SigmoidMoe(_Module):
         super().__init__(model)
         self.s, self.p = spec, prefix
 
+    wants_f32_input = True
+
     def load(self, get):
         s, p, m = self.s, self.p, self.m
         dev, dt = m.device, m.torch_dtype
@@ -558,6 +660,7 @@ class ClampedSoftmaxMoe(_Module):
     biases): g = min(gate h, limit), u = clamp(up h, -limit, limit), down(g sigmoid(1.702 g) (u + 1)); a shared expert of the same form (its own size and limit) runs for
     every row with weight 1.  All experts of a step run as grouped products over expert-sorted rows."""
     ALPHA = 1.702
+    wants_f32_input = True
 
     def __init__(self, model, spec: ClampedMoeSpec, prefix: str):
         super().__init__(model)
@@ -643,8 +746,204 @@ class XieluFeedForward(_Module):
         m.linear(a, self.w_down, out=x, accumulate=accumulate)
 
 
-MIXERS: Dict[str, Callable] = {"mamba2": Mamba2Mixer, "attention": WindowAttention, "talk_attention": TalkSigmoidAttention}
-FEED_FORWARDS: Dict[str, Callable] = {"moe": SigmoidMoe, "moe_softmax_clamped": ClampedSoftmaxMoe, "dense_xielu": XieluFeedForward}
+class GatedSinkAttention(_Module):
+    """q, k, v (with biases) and the gate logits in one product; an optional short causal convolution over every q / k / v channel (no bias, no activation; the last
+    taps - 1 projected rows ride in the sequence's state slot); no rotation: positions enter through a query temperature (q *= 1 + coef ln(floor((pos + 1) / every) + 1)).
+    Score s = scale (q . k), optionally cap tanh(s / cap); causal softmax with a sink, p_j = e^{s_j} / (1 + sum e^{s}); the concatenated heads times sigmoid(gate logits)
+    element by element, then the output projection.  With `kv_from` the layer has no key / value projections: it reads the K / V pages of that earlier layer."""
+
+    def __init__(self, model, spec: SinkAttentionSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        if spec.heads % spec.kv_heads:
+            raise ValueError(f"{prefix}: heads % kv_heads must be 0")
+        dev, bs, nb = model.device, model.block_size, model.num_blocks
+        self.own = spec.kv_from is None
+        self.k_cache = self.v_cache = None
+        if self.own:
+            self.k_cache = torch.zeros(nb, spec.kv_heads, bs, spec.dim, dtype=model.torch_dtype, device=dev)
+            self.v_cache = torch.zeros(nb, spec.kv_heads, bs, spec.vdim, dtype=model.torch_dtype, device=dev)
+        self.nq, self.nk, self.nv = spec.heads * spec.dim, spec.kv_heads * spec.dim, spec.kv_heads * spec.vdim
+        self.channels = self.nq + (self.nk + self.nv if self.own else 0)
+        self.conv_state = torch.zeros(model.state_slots, self.channels, spec.conv - 1, dtype=torch.float32, device=dev) if spec.conv > 1 else None
+
+    def carried(self):
+        return tuple(t for t in (self.k_cache, self.v_cache, self.conv_state) if t is not None)
+
+    def kv_bytes_per_token(self) -> int:
+        return self.k_cache.element_size() * self.s.kv_heads * (self.s.dim + self.s.vdim) if self.own else 0
+
+    def state_bytes_per_slot(self) -> int:
+        return 4 * self.conv_state[0].numel() if self.conv_state is not None else 0
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        names = ["q", "k", "v"] if self.own else ["q"]
+        parts = [get(p + n) for n in names] + [get(p + "g")]
+        want = [self.nq, self.nk, self.nv][:len(names)] + [s.heads * s.vdim]
+        if [t.shape[0] for t in parts] != want or any(t.shape[1] != W for t in parts):
+            raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
+        self.w_in = torch.cat(parts, 0).to(self.m.device, self.m.torch_dtype).contiguous()     # [q | k | v | gate, W]
+        self.gate_col = self.channels
+        self.bias = torch.cat([get(p + n + ".b").reshape(-1) for n in names], 0).to(self.m.device, torch.float32).contiguous()   # [q | k | v]
+        self.conv_w = None
+        if s.conv:
+            self.conv_w = torch.cat([get(p + n + ".conv") for n in names], 0).to(self.m.device, torch.float32).contiguous()     # [channels, taps]
+            if tuple(self.conv_w.shape) != (self.channels, s.conv):
+                raise ValueError(f"{p}: convolution shapes do not match the mixer's sizes")
+        self.w_o = self.w(get, p + "o", True)
+        if self.bias.numel() != self.channels or tuple(self.w_o.shape) != (W, s.heads * s.vdim):
+            raise ValueError(f"{p}: bias / output shapes do not match the mixer's sizes")
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T = b.rows
+        u = m.linear(h, self.w_in)                                         # f32 [T, q | k | v | gate logits]
+        qb = self.bias[:self.nq]
+        kb, vb = (self.bias[self.nq:self.nq + self.nk], self.bias[self.nq + self.nk:]) if self.own else (None, None)
+        src_rows, ld = u, u.stride(0)
+        if s.conv:
+            src_rows = torch.empty(T, self.channels, dtype=torch.float32, device=m.device)
+            _call("mrs_hyb_conv", u, u.stride(0), self.bias, self.conv_w, None, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, src_rows, T, b.entries,
+                  self.channels, s.conv, 0)
+            ld, qb, kb, vb = self.channels, None, None, None
+        q = torch.empty(T, self.nq, dtype=m.torch_dtype, device=m.device)
+        _call("mrs_hyb_qkv_bias_temp_cache", src_rows, ld, qb, kb, vb, b.tok_pos, b.slot_mapping, q, self.k_cache, self.v_cache, T, s.heads, s.kv_heads, s.dim, s.vdim,
+              m.block_size, s.temp_coef, s.temp_every, m.dt)
+        src = self if self.own else m.layers[s.kv_from].mixer               # that layer ran earlier in this step: its pages hold this step's rows already
+        o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
+        _call("mrs_hyb_paged_attn_opts", q, src.k_cache, src.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, b.max_blocks,
+              0, 0, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, s.softcap, int(s.sink), u[:, self.gate_col:], u.stride(0))
+        m.linear(o, self.w_o, out=x, accumulate=accumulate)
+
+
+class RetentionMixer(_Module):
+    """v | k | q | gate in one product (no biases); half-split rotary on the first `rot.dims` dimensions of every query and key head (angles from f32 positions), keys
+    times dim^(-1/2); per head the f32 state S [dim, vdim] <- decay_h S + k v^T and o = S^T q, carried per sequence slot; o / rms(o) per head (no weight), times
+    silu(gate), output projection.  The recurrence is the state-space scan with unit steps and fixed decays (segments of a long portion run in parallel)."""
+
+    def __init__(self, model, spec: RetentionSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        if spec.rotary and spec.rotary.layout != "half":
+            raise ValueError(f"{prefix}: retention rotates half-split pairs")
+        dev = model.device
+        self.state = torch.zeros(model.state_slots, spec.heads, spec.dim, spec.vdim, dtype=torch.float32, device=dev)
+        self.decay = torch.tensor(spec.decay, dtype=torch.float64).to(dev, torch.float32)
+        self.freq = torch.from_numpy(spec.rotary.frequencies()).to(dev) if spec.rotary else None
+        self.k_mult = float(np.float32(spec.dim) ** np.float32(-0.5))
+
+    def carried(self):
+        return (self.state,)
+
+    def state_bytes_per_slot(self) -> int:
+        return 4 * self.state[0].numel()
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        parts = [get(p + n) for n in ("v", "k", "q", "g")]
+        want = [s.heads * s.vdim, s.heads * s.dim, s.heads * s.dim, s.heads * s.vdim]
+        if [t.shape[0] for t in parts] != want or any(t.shape[1] != W for t in parts):
+            raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
+        self.w_in = torch.cat(parts, 0).to(self.m.device, self.m.torch_dtype).contiguous()     # [v | k | q | gate, W]
+        self.k_col, self.q_col, self.gate_col = want[0], want[0] + want[1], want[0] + 2 * want[1]
+        self.w_o = self.w(get, p + "o", True)
+        if tuple(self.w_o.shape) != (W, s.heads * s.vdim):
+            raise ValueError(f"{p}: output shape does not match the mixer's sizes")
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T, dev = b.rows, m.device
+        u = m.linear(h, self.w_in)                                         # f32 [T, v | k | q | gate]
+        _call("mrs_hyb_rotary_half", u, u.stride(0), self.q_col, self.k_col, s.heads, s.dim, s.rotary.dims if s.rotary else 0, self.freq, b.tok_pos, self.k_mult, T)
+        y = torch.empty(T, s.heads * s.vdim, dtype=torch.float32, device=dev)
+        steps = torch.empty(T, s.heads, 2, dtype=torch.float32, device=dev)
+        carry = decay = None
+        if b.segments > b.entries:   # some portion is longer than a segment: scratch for the segments' local end states
+            carry = torch.empty(b.segments, s.heads, s.dim, s.vdim, dtype=torch.float32, device=dev)
+            decay = torch.empty(b.segments, s.heads, dtype=torch.float32, device=dev)
+        _call("mrs_hyb_decay_scan", u, u.stride(0), self.decay, self.state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, steps, carry, decay,
+              T, b.entries, b.segments, s.heads, s.vdim, s.dim, s.heads)
+        yn = m.norm(y, None, one_plus=False, parts=s.heads, gate=u[:, self.gate_col:], gate_after=True)   # per-head unit norm, then silu(gate)
+        m.linear(yn, self.w_o, out=x, accumulate=accumulate)
+
+
+class LatentAttention(_Module):
+    """q | latent in one product; the latent row c = norm(W_dkv h) (plain weight) is the only thing paged.  Head h's keys W_uk,h c and values W_uv,h c are never
+    materialised: q'_h = W_uk,h^T q_h scores against the cached rows (one shared key / value head of kv_rank dimensions for all query heads), the weighted sum of cached
+    rows is expanded by W_uv,h afterwards -- the same sums, reassociated.  Causal softmax, s = scale (q . k); no positions."""
+
+    def __init__(self, model, spec: LatentAttentionSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        self.c_cache = torch.zeros(model.num_blocks, 1, model.block_size, spec.kv_rank, dtype=model.torch_dtype, device=model.device)
+
+    def carried(self):
+        return (self.c_cache,)
+
+    def kv_bytes_per_token(self) -> int:
+        return self.c_cache.element_size() * self.s.kv_rank
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        dev, dt = self.m.device, self.m.torch_dtype
+        q, dkv, uk, uv = (get(p + n) for n in ("q", "dkv", "uk", "uv"))
+        if tuple(q.shape) != (s.heads * s.dim, W) or tuple(dkv.shape) != (s.kv_rank, W) or tuple(uk.shape) != (s.heads * s.dim, s.kv_rank) or \
+                tuple(uv.shape) != (s.heads * s.vdim, s.kv_rank):
+            raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
+        self.w_in = torch.cat([q, dkv], 0).to(dev, dt).contiguous()                                       # [q | latent, W]
+        self.w_ukT = uk.reshape(s.heads, s.dim, s.kv_rank).transpose(1, 2).to(dev, dt).contiguous()       # [H, kv_rank, dim]: q' = this . q
+        self.w_uv = uv.reshape(s.heads, s.vdim, s.kv_rank).to(dev, dt).contiguous()                       # [H, vdim, kv_rank]
+        self.c_norm = self.w(get, p + "dkv.norm", False)
+        self.w_o = self.w(get, p + "o", True)
+        if self.c_norm.numel() != s.kv_rank or tuple(self.w_o.shape) != (W, s.heads * s.vdim):
+            raise ValueError(f"{p}: norm / output shapes do not match the mixer's sizes")
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T, dev, dt = b.rows, m.device, m.torch_dtype
+        H, D, Dv, R = s.heads, s.dim, s.vdim, s.kv_rank
+        u = m.linear(h, self.w_in)                                         # f32 [T, q | latent]
+        q = torch.empty(T, H * D, dtype=dt, device=dev)
+        _call("mrs_hyb_latent_norm_cache", u, u.stride(0), H * D, R, self.c_norm, b.slot_mapping, q, self.c_cache, m.spec.eps, T, m.dt)
+        qa = m.batched_linear(q, self.w_ukT, H)                            # [T, H * kv_rank] in the serving dtype
+        oa = torch.empty(T, H * R, dtype=dt, device=dev)
+        _call("mrs_hyb_paged_attn_opts", qa, self.c_cache, self.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, m.block_size, b.max_blocks, 0, 0, s.scale,
+              m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, 0, None, 0)
+        ov = m.batched_linear(oa, self.w_uv, H)                            # [T, H * vdim]
+        m.linear(ov, self.w_o, out=x, accumulate=accumulate)
+
+
+class GluFeedForward(_Module):
+    """down(silu(gate h) * (up h)), no biases; gate | up are one product."""
+
+    def __init__(self, model, spec: GluSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        g, u = get(p + "gate"), get(p + "up")
+        self.w_down = self.w(get, p + "down", True)
+        if tuple(g.shape) != (s.ff, W) or tuple(u.shape) != (s.ff, W) or tuple(self.w_down.shape) != (W, s.ff):
+            raise ValueError(f"{p}: projection shapes do not match the layer's sizes")
+        self.w_gu = torch.cat([g, u], 0).to(self.m.device, self.m.torch_dtype).contiguous()
+
+    def forward(self, h, h32, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T = b.rows
+        gu = m.linear(h, self.w_gu)
+        if T <= m.GEMV_ROWS:   # decode-sized steps: the GLU in the down product's operand load
+            _call("mrs_hyb_gemv", gu, self.w_down, x, T, x.shape[1], s.ff, 2 * s.ff, s.ff, x.stride(0), m.dt, int(accumulate), None, 0, 1, None, None, 1)
+            return
+        a = torch.empty(T, s.ff, dtype=m.torch_dtype, device=m.device)
+        _call("mrs_hyb_glu_silu", gu, a, T, s.ff, m.dt)
+        m.linear(a, self.w_down, out=x, accumulate=accumulate)
+
+
+MIXERS: Dict[str, Callable] = {"mamba2": Mamba2Mixer, "attention": WindowAttention, "talk_attention": TalkSigmoidAttention, "sink_attention": GatedSinkAttention,
+                               "retention": RetentionMixer, "latent_attention": LatentAttention}
+FEED_FORWARDS: Dict[str, Callable] = {"moe": SigmoidMoe, "moe_softmax_clamped": ClampedSoftmaxMoe, "dense_xielu": XieluFeedForward, "dense_glu_silu": GluFeedForward}
 
 
 class _Layer:
@@ -653,6 +952,7 @@ class _Layer:
         self.mixer = MIXERS[ls.kind](model, ls.mixer, ls.prefix + "mix.")
         self.ff = FEED_FORWARDS[ls.ff.kind](model, ls.ff, ls.prefix + "mlp.") if ls.ff else None
         self.norm1 = self.norm2 = self.norm1b = self.norm2b = None   # (weight, bias | None)
+        self.hc1 = self.hc2 = None   # several residual streams: (in [S], out [S] times the residual multiplier, mix [S, S]) of the sublayer, f32
 
 
 # ------------------------------------------------------------------------------------------------------------------ the model
@@ -676,7 +976,7 @@ class HybridDecoder:
     # ---- construction
     @property
     def has_recurrent_state(self) -> bool:
-        return any(isinstance(l.mixer, Mamba2Mixer) for l in self.layers)
+        return self.state_bytes_per_slot() > 0
 
     @property
     def has_paged_kv(self) -> bool:
@@ -691,7 +991,23 @@ class HybridDecoder:
         self.final_norm = norm(sp.final_norm)
         if tuple(self.embed.shape) != (sp.vocab, sp.width) or tuple(self.head.shape) != (sp.vocab, sp.width):
             raise ValueError("embedding / head shapes do not match vocab x width")
+        self.embed_norm = norm(sp.embed_norm) if sp.embed_norm else None
+        S = max(1, sp.streams)
+        self.ones = torch.ones(S, dtype=torch.float32, device=self.device)
+
+        def hyper(prefix):
+            """(in, residual_mult * out, mix) of a sublayer; one plain stream: (1, residual_mult, 1)"""
+            if not sp.streams:
+                return self.ones, torch.full((1,), sp.residual_mult, dtype=torch.float32, device=self.device), self.ones.view(1, 1)
+            w_in, w_out, mix = f32(prefix + ".in").reshape(-1), f32(prefix + ".out").reshape(-1), f32(prefix + ".mix")
+            if w_in.numel() != S or w_out.numel() != S or tuple(mix.shape) != (S, S):
+                raise ValueError(f"{prefix}: stream weights do not match the number of streams")
+            return w_in, (w_out * np.float32(sp.residual_mult)).contiguous(), mix
+        self.multi_stream = bool(sp.streams) or sp.residual_mult != 1.0
         for l in self.layers:
+            if self.multi_stream:
+                l.hc1 = hyper(l.spec.prefix + "hc1")
+                l.hc2 = hyper(l.spec.prefix + "hc2") if l.ff else None
             l.norm1 = norm(l.spec.prefix + "norm1")
             l.norm1b = norm(l.spec.prefix + "norm1b") if sp.post_norms else None
             l.mixer.load(get)
@@ -712,13 +1028,35 @@ class HybridDecoder:
         return model
 
     # ---- building blocks on the current stream
-    def norm(self, x, w, one_plus: bool, parts: int = 1, want32: bool = False, gate=None):
-        """RMS norm of every row (in `parts` equal pieces); gate [rows, >= width]: the row is multiplied by silu(gate) first."""
+    def norm(self, x, w, one_plus: bool, parts: int = 1, want32: bool = False, gate=None, gate_after: bool = False):
+        """RMS norm of every row (in `parts` equal pieces; w None: no weight); gate [rows, >= width]: the row is multiplied by silu(gate) first, or (gate_after) the
+        normed row is."""
         rows, width = x.shape
         out = torch.empty(rows, width, dtype=self.torch_dtype, device=self.device)
         out32 = torch.empty(rows, width, dtype=torch.float32, device=self.device) if want32 else None
-        _call("mrs_hyb_rmsnorm", x, x.stride(0), w, out, out32, None, rows, width, parts, self.spec.eps, int(one_plus), self.dt, gate, gate.stride(0) if gate is not None else 0)
+        _call("mrs_hyb_rmsnorm", x, x.stride(0), w, out, out32, None, rows, width, parts, self.spec.eps, int(one_plus), self.dt, gate, gate.stride(0) if gate is not None else 0,
+              int(gate_after))
         return (out, out32) if want32 else out
+
+    def hyper_step(self, x, y, write, read, norm_w, want32: bool = False):
+        """One launch between two sublayers of a design with residual streams x [rows, S, W]: `write` = (_, out, mix) of the sublayer that made y (mix None: the streams
+        start as out[r] * y), `read` = the in-weights of the next reader, `norm_w` its one-plus norm weight (None: the read sum itself comes back in f32)."""
+        rows, S, W = x.shape
+        out = torch.empty(rows, W, dtype=self.torch_dtype, device=self.device) if norm_w is not None else None
+        out32 = torch.empty(rows, W, dtype=torch.float32, device=self.device) if (want32 or norm_w is None) else None
+        _call("mrs_hyb_hyper_step", x, y, write[2] if y is not None else None, write[1] if y is not None else None, read, norm_w, out, out32, rows, S, W, self.spec.eps, 1, self.dt)
+        if norm_w is None:
+            return out32
+        return (out, out32) if want32 else out
+
+    def batched_linear(self, a, w, heads: int):
+        """a [M, heads * K] (column block h = the operand of head h), w [heads, N, K] -> [M, heads * N] in the serving dtype, rounded once: per-head products whose
+        consumer is another product or the attention kernel."""
+        M = a.shape[0]
+        _, N, K = w.shape
+        out = torch.empty(M, heads * N, dtype=self.torch_dtype, device=self.device)
+        _call("mrs_hyb_gemm_batched", a, w, out, M, N, K, a.stride(0), K, out.stride(0), self.dt, heads, K, N * K, N, 1)
+        return out
 
     def layer_norm(self, x, wb, want32: bool = False):
         """(x - mean) / sqrt(var + eps) * w + b of every row, in the serving dtype (and in f32 with want32)."""
@@ -795,6 +1133,15 @@ class HybridDecoder:
             return torch.empty(0, sp.vocab, dtype=torch.float32, device=self.device)
         x = torch.empty(T, sp.width, dtype=torch.float32, device=self.device)
         _call("mrs_hyb_embed", b.tokens, self.embed, x, T, sp.width, sp.vocab, self.dt)
+        if self.embed_norm is not None:
+            e = torch.empty_like(x)
+            if sp.norm == "layer":
+                _call("mrs_hyb_layernorm", x, x.stride(0), None, self.embed_norm[0], self.embed_norm[1], None, e, None, 0, T, sp.width, sp.eps, self.dt)
+            else:
+                _call("mrs_hyb_rmsnorm", x, x.stride(0), self.embed_norm[0], None, e, None, T, sp.width, 1, sp.eps, 1, self.dt, None, 0, 0)
+            x = e
+        if self.multi_stream:
+            return self._forward_streams(b, x)
         y = torch.empty_like(x) if sp.post_norms else None   # a sublayer's product on its way through the norm behind it
         h_next = None                                         # post-norm designs: the next sublayer's input, normed by the launch that closed the previous sublayer
         for li, l in enumerate(self.layers):
@@ -821,6 +1168,42 @@ class HybridDecoder:
         _call("mrs_hyb_gather_rows", x, b.want, xs, n, sp.width)
         return self.linear(self.pre_norm(xs, self.final_norm), self.head)
 
+    def _forward_streams(self, b: RaggedBatch, e: torch.Tensor) -> torch.Tensor:
+        """Designs with scaled sublayer outputs and / or several residual streams: x [rows, S, W] f32.  Every sublayer's product goes to a scratch block; the launch that
+        writes it into the streams also reads and norms the input of the NEXT sublayer, so a sublayer costs one launch besides its own."""
+        sp = self.spec
+        if sp.post_norms or sp.norm != "rms_one_plus":
+            raise NotImplementedError("residual streams are built for one-plus RMS norms in front of the sublayers")
+        T, W, S = b.rows, sp.width, max(1, sp.streams)
+        subs = []   # (layer, module, (in, out, mix), norm weight, last sublayer of its layer)
+        for l in self.layers:
+            subs.append((l, l.mixer, l.hc1, l.norm1[0], l.ff is None))
+            if l.ff:
+                subs.append((l, l.ff, l.hc2, l.norm2[0], True))
+        x = torch.empty(T, S, W, dtype=torch.float32, device=self.device)
+        y = torch.empty(T, W, dtype=torch.float32, device=self.device)
+        h = self.hyper_step(x, e, (None, self.ones, None), subs[0][2][0], subs[0][3], want32=subs[0][1].wants_f32_input)
+        total = None
+        for k, (l, mod, hc, _, closes) in enumerate(subs):
+            if mod is l.mixer:
+                mod.forward(h, y, b, accumulate=False)
+            else:
+                h, h32 = h if isinstance(h, tuple) else (h, None)
+                mod.forward(h, h32, y, b, accumulate=False)
+            if k + 1 < len(subs):
+                nxt = subs[k + 1]
+                h = self.hyper_step(x, y, hc, nxt[2][0], nxt[3], want32=nxt[1].wants_f32_input)
+            else:
+                total = self.hyper_step(x, y, hc, self.ones, None)   # the sum of the streams
+            if closes and self.trace_layers is not None:
+                self.trace_layers.append(x.sum(1))
+        n = b.want.numel()
+        if n == 0:
+            return torch.empty(0, sp.vocab, dtype=torch.float32, device=self.device)
+        xs = torch.empty(n, W, dtype=torch.float32, device=self.device)
+        _call("mrs_hyb_gather_rows", total, b.want, xs, n, W)
+        return self.linear(self.pre_norm(xs, self.final_norm), self.head)
+
     # ---- decode steps as a HIP graph
     def capture_decode(self, entries: int, max_blocks: int) -> "DecodeGraph":
         """One decode step for `entries` sequences (one row each), captured into a HIP graph over static batch buffers: replays cost one launch instead of one per kernel."""
@@ -831,7 +1214,7 @@ class HybridDecoder:
         return sum(l.mixer.kv_bytes_per_token() for l in self.layers if hasattr(l.mixer, "kv_bytes_per_token"))
 
     def state_bytes_per_slot(self) -> int:
-        return sum(l.mixer.state_bytes_per_slot() for l in self.layers if isinstance(l.mixer, Mamba2Mixer))
+        return sum(l.mixer.state_bytes_per_slot() for l in self.layers if hasattr(l.mixer, "state_bytes_per_slot"))
 
 
 class DecodeGraph:
@@ -960,7 +1343,7 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
     return get
 
 
-SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec, "Sobunex": sobunex_spec}
+SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec, "Sobunex": sobunex_spec, "Setopel": setopel_spec}
 
 
 class HybridCache:
