@@ -980,7 +980,7 @@ class HybridDecoder:
 
     @property
     def has_paged_kv(self) -> bool:
-        return any(hasattr(l.mixer, "k_cache") for l in self.layers)
+        return self.kv_bytes_per_token() > 0
 
     def load_weights(self, get: Callable[[str], torch.Tensor]) -> None:
         sp = self.spec
@@ -1283,12 +1283,29 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
     W = spec.width
     g = torch.Generator(device=device).manual_seed(seed)
     shapes: Dict[str, tuple] = {spec.embed: (spec.vocab, W), spec.head: (spec.vocab, W), spec.final_norm: (W,)}
-    norm_names = {spec.final_norm}
+    norm_names = {spec.final_norm} | ({spec.embed_norm} if spec.embed_norm else set())
     for ls in spec.layers:
         p, m = ls.prefix, ls.mixer
         for n in ["norm1"] + (["norm2"] if ls.ff else []) + ((["norm1b"] + (["norm2b"] if ls.ff else [])) if spec.post_norms else []):
             norm_names.add(p + n)
-        if isinstance(m, TalkAttentionSpec):
+        if spec.streams:
+            for q in ("hc1", "hc2") if ls.ff else ("hc1",):
+                shapes.update({f"{p}{q}.in": (spec.streams,), f"{p}{q}.out": (spec.streams,), f"{p}{q}.mix": (spec.streams, spec.streams)})
+        if isinstance(m, SinkAttentionSpec):
+            own = ["q", "k", "v"] if m.kv_from is None else ["q"]
+            rows = {"q": m.heads * m.dim, "k": m.kv_heads * m.dim, "v": m.kv_heads * m.vdim}
+            for n in own:
+                shapes.update({f"{p}mix.{n}": (rows[n], W), f"{p}mix.{n}.b": (rows[n],)})
+                if m.conv:
+                    shapes[f"{p}mix.{n}.conv"] = (rows[n], m.conv)
+            shapes.update({p + "mix.g": (m.heads * m.vdim, W), p + "mix.o": (W, m.heads * m.vdim)})
+        elif isinstance(m, RetentionSpec):
+            shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.heads * m.dim, W), p + "mix.v": (m.heads * m.vdim, W), p + "mix.g": (m.heads * m.vdim, W),
+                           p + "mix.o": (W, m.heads * m.vdim)})
+        elif isinstance(m, LatentAttentionSpec):
+            shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.dkv": (m.kv_rank, W), p + "mix.dkv.norm": (m.kv_rank,), p + "mix.uk": (m.heads * m.dim, m.kv_rank),
+                           p + "mix.uv": (m.heads * m.vdim, m.kv_rank), p + "mix.o": (W, m.heads * m.vdim)})
+        elif isinstance(m, TalkAttentionSpec):
             shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.q.b": (m.heads * m.dim,), p + "mix.g": (m.heads, W), p + "mix.talk": (m.heads, m.heads),
                            p + "mix.pb": (m.heads,), p + "mix.o": (W, m.heads * m.vdim), p + "mix.o.b": (W,)})
             if m.kv_from is None:
@@ -1299,7 +1316,9 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
         else:
             shapes.update({p + "mix.q": (m.heads * m.dim, W), p + "mix.k": (m.kv_heads * m.dim, W), p + "mix.v": (m.kv_heads * m.vdim, W), p + "mix.q.norm": (m.heads * m.dim,),
                            p + "mix.k.norm": (m.kv_heads * m.dim,), p + "mix.o": (W, m.heads * m.vdim)})
-        if isinstance(ls.ff, DenseSpec):
+        if isinstance(ls.ff, GluSpec):
+            shapes.update({p + "mlp.gate": (ls.ff.ff, W), p + "mlp.up": (ls.ff.ff, W), p + "mlp.down": (W, ls.ff.ff)})
+        elif isinstance(ls.ff, DenseSpec):
             shapes.update({p + "mlp.up": (ls.ff.ff, W), p + "mlp.up.b": (ls.ff.ff,), p + "mlp.down": (W, ls.ff.ff), p + "mlp.down.b": (W,), p + "mlp.act": (2,)})
         elif ls.ff:
             f = ls.ff
@@ -1319,7 +1338,13 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
         shape = shapes[name]
         r = torch.randn(*shape, device=device, generator=g)
         last = name.rsplit(".", 1)[-1]
-        if name.endswith(("q.norm", "k.norm")) or last == "D" or name.endswith("mix.norm") or (name in norm_names and spec.norm == "layer"):
+        if name.endswith(("q.norm", "k.norm", "dkv.norm")) or last == "D" or name.endswith("mix.norm") or (name in norm_names and spec.norm == "layer"):
+            r = 1.0 + 0.1 * r
+        elif last == "mix" and len(shape) == 2 and shape[0] == shape[1] == spec.streams:
+            r = torch.eye(shape[0], device=device) + 0.1 * r
+        elif last == "in" and shape == (spec.streams,):
+            r = 1.0 / spec.streams + 0.1 * r
+        elif last == "out" and shape == (spec.streams,):
             r = 1.0 + 0.1 * r
         elif name in norm_names:
             r = 0.1 * r
