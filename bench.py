@@ -846,6 +846,199 @@ def sobunex_leg(a, dev):
                       "ms_per_step": d1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
                       "config": {"model": f"sobunex-{a.sobunex}", "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "sobunex": out}), flush=True)
 
+SETOPEL_SIZES = {
+    # layer lists that resemble a small, a mid-size and a large decoder: latent attention, sink attention (every second one reads the pages of the first) and retention in turn
+    "s": dict(width=1024, layers=8, heads=16, kv=4, dim=64, vdim=64, rank=256, ret_heads=8, ret_dim=64, ret_vdim=128, ff=2816, streams=4, conv=4, vocab=32000),
+    "m": dict(width=2048, layers=8, heads=16, kv=4, dim=128, vdim=128, rank=512, ret_heads=8, ret_dim=128, ret_vdim=256, ff=5632, streams=4, conv=4, vocab=32000),
+    "l": dict(width=4096, layers=4, heads=32, kv=8, dim=128, vdim=128, rank=512, ret_heads=16, ret_dim=128, ret_vdim=256, ff=11008, streams=4, conv=4, vocab=32000),
+}
+
+
+def setopel_leg(a, dev):
+    """`--setopel SIZE`: prefill and decode throughput of a Setopel layer list (residual streams; latent attention, sink attention with convolved projections, retention;
+    SiLU-GLU feed-forwards; bf16 weights, random) beside the closest model of the package at equal size: a list of rotary softmax attention layers (in place of the two
+    attention kinds) and state-space layers (in place of retention, equal state size) with dense feed-forwards of equal weight bytes and one residual stream.  Then the
+    kernels of the two designs that do like work, one launch each at the model's shapes: time and the fraction of the roofline (8 TB/s for what a kernel must read and
+    write; prompt attention and the recurrences run on the f32 vector ALU in both designs and are priced in FLOP/s of the work done)."""
+    import torch
+    from mistralrs_amd.hybrid import (AttentionSpec, DenseSpec, GluSpec, HybridCache, HybridDecoder, HybridSpec, LatentAttentionSpec, LayerSpec, Mamba2Spec, RaggedBatch,
+                                      RetentionSpec, RotarySpec, SinkAttentionSpec, _call, synthetic_weights)
+    z = SETOPEL_SIZES[a.setopel]
+    W, H, G, D, Dv, R = z["width"], z["heads"], z["kv"], z["dim"], z["vdim"], z["rank"]
+    rh, rd, rv = z["ret_heads"], z["ret_dim"], z["ret_vdim"]
+    new_layers, old_layers = [], []
+    first_attn = None
+    for i in range(z["layers"]):
+        kind = ("latent", "attention", "retention")[i % 3]
+        if kind == "latent":
+            new_layers.append(LayerSpec("latent_attention", LatentAttentionSpec(H, D, Dv, R, D ** -0.5), GluSpec(z["ff"]), f"l{i}."))
+        elif kind == "attention":
+            src = first_attn if first_attn is not None and (i // 3) % 2 == 1 else None
+            new_layers.append(LayerSpec("sink_attention", SinkAttentionSpec(H, G, D, Dv, D ** -0.5, z["conv"], 30.0, 0.25, 256, src), GluSpec(z["ff"]), f"l{i}."))
+            first_attn = i if first_attn is None else first_attn
+        else:
+            decay = [1.0 - 2.0 ** (-5 - (7.0 * h) / max(1, rh - 1)) for h in range(rh)]
+            new_layers.append(LayerSpec("retention", RetentionSpec(rh, rd, rv, decay, RotarySpec(rd, 10000.0, None, "half")), None, f"l{i}."))
+        if kind == "retention":
+            old_layers.append(LayerSpec("mamba2", Mamba2Spec(rh, rv, rd, rh, z["conv"], 1), None, f"l{i}."))
+        else:
+            old_layers.append(LayerSpec("attention", AttentionSpec(H, G, D, Dv, D ** -0.5, 0, 0, RotarySpec(D // 2, 500000.0, None)), DenseSpec(3 * z["ff"] // 2), f"l{i}."))
+    specs = {"setopel": HybridSpec(z["vocab"], W, 1e-6, new_layers, embed_norm="embed.norm", residual_mult=0.5, streams=z["streams"]),
+             "attention_state_space_dense": HybridSpec(z["vocab"], W, 1e-6, old_layers)}
+    prompts, batches, bs, ctx = [512, 2048], [1, 8], 32, 512
+    max_tok = max(prompts) + a.warmup + a.steps + 64
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    out = {"sizes": z, "dtype": "bf16", "weights": "random, drawn on the device", "models": {}, "kernels": {}}
+    keep = {}
+    with torch.no_grad():
+        for name, spec in specs.items():
+            model = HybridDecoder(spec, dev, "bfloat16", num_blocks=max(batches) * (-(-max_tok // bs) + 1) + 2, block_size=bs, state_slots=max(batches))
+            model.load_weights(synthetic_weights(spec, dev, 0))
+            cache = HybridCache(model)
+            r = {"prefill": {}, "decode": {}}
+            for T in prompts:
+                assert cache.reserve(1, T)
+                b = RaggedBatch.build([cache.entry(1, [(1000 + i) % z["vocab"] for i in range(T)], 0, [T - 1])], bs, dev)
+                t = timed(lambda: model.forward_batch(b), 3)
+                r["prefill"][str(T)] = {"tokens_per_sec": round(T / t, 1), "ms": round(1e3 * t, 3)}
+                cache.release(1)
+            for nb in batches:
+                for q in range(nb):
+                    assert cache.reserve(q + 1, ctx + a.warmup + a.steps + 2)
+                model.forward_batch(RaggedBatch.build([cache.entry(q + 1, [(1000 + i + q) % z["vocab"] for i in range(ctx)], 0, []) for q in range(nb)], bs, dev))
+                g = model.capture_decode(nb, -(-(ctx + a.warmup + a.steps + 2) // bs))
+                pos = ctx
+
+                def step():
+                    nonlocal pos
+                    g.replay([cache.entry(q + 1, [7 + q], pos) for q in range(nb)])
+                    pos += 1
+                for _ in range(a.warmup):
+                    step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(a.steps):
+                    step()
+                torch.cuda.synchronize()
+                t = (time.perf_counter() - t0) / a.steps
+                r["decode"][f"batch{nb}"] = {"tokens_per_sec": round(nb / t, 1), "ms_per_step": round(1e3 * t, 4)}
+                del g
+                for q in range(nb):
+                    cache.release(q + 1)
+            out["models"][name] = r
+            keep[name] = model
+            torch.cuda.empty_cache()
+        # ---- like kernels of the two designs, one launch each
+        new, old = keep["setopel"], keep["attention_state_space_dense"]
+        kern = out["kernels"]
+        e = 2
+        bps = -(-(2048 + 64) // bs)
+
+        def pair(label, t_new, t_old, nbytes=None, flops=None, **extra):
+            d = {"setopel_us": round(1e6 * t_new, 1), "other_us": round(1e6 * t_old, 1), "time_ratio": round(t_new / t_old, 2), **extra}
+            if nbytes is not None:
+                d.update(min_bytes=nbytes[0], other_min_bytes=nbytes[1], setopel_hbm_frac=round(nbytes[0] / t_new / HBM_PEAK, 4), other_hbm_frac=round(nbytes[1] / t_old / HBM_PEAK, 4))
+            if flops is not None:
+                d.update(flops=flops[0], other_flops=flops[1], setopel_tflops=round(flops[0] / t_new / 1e12, 2), other_tflops=round(flops[1] / t_old / 1e12, 2))
+            kern[label] = d
+        sink, latent, retn = new.layers[1].mixer, new.layers[0].mixer, new.layers[2].mixer
+        oattn, ossm = old.layers[1].mixer, old.layers[2].mixer
+        for c in (sink.k_cache, sink.v_cache, oattn.k_cache, oattn.v_cache, latent.c_cache):
+            c.normal_()
+        for label, nseq, p0, n in (("attention_prompt_2048", 1, 0, 2048), ("attention_decode_batch8_ctx2048", 8, 2047, 1), ("attention_decode_batch1_ctx2048", 1, 2047, 1)):
+            ents = [{"tokens": [0] * n, "pos0": p0, "slot": 0, "blocks": list(range(1 + q * bps, 1 + (q + 1) * bps)), "want": []} for q in range(nseq)]
+            if ents[-1]["blocks"][-1] >= new.num_blocks:
+                continue
+            b = RaggedBatch.build(ents, bs, dev)
+            T = b.rows
+            qn = torch.randn(T, H * D, device=dev).to(torch.bfloat16)
+            gate = torch.randn(T, H * Dv, device=dev)
+            o = torch.empty(T, H * Dv, dtype=torch.bfloat16, device=dev)
+            seg = (b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
+            t_new = timed(lambda: _call("mrs_hyb_paged_attn_opts", qn, sink.k_cache, sink.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, 0, 0,
+                                        D ** -0.5, 1, *seg, 30.0, 1, gate, H * Dv, *new.key_splits(b, H, Dv)), 5)
+            t_old = timed(lambda: _call("mrs_hyb_paged_window_attn", qn, oattn.k_cache, oattn.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, 0, 0,
+                                        D ** -0.5, 1, *seg), 5)
+            pairs = sum(p0 + i + 1 for i in range(n)) * nseq
+            fl = 2.0 * pairs * H * (D + Dv)
+            kvb = nseq * e * G * (D + Dv) * (p0 + n) + T * e * H * (D + Dv)
+            pair("sink_" + label, t_new, t_old, (kvb + T * H * Dv * 4, kvb), (fl, fl))
+            # latent attention: the same kernel, one shared head of `rank` dimensions for keys and values
+            qa = torch.randn(T, H * R, device=dev).to(torch.bfloat16)
+            oa = torch.empty(T, H * R, dtype=torch.bfloat16, device=dev)
+            t_lat = timed(lambda: _call("mrs_hyb_paged_attn_opts", qa, latent.c_cache, latent.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, bs, b.max_blocks, 0, 0,
+                                        D ** -0.5, 1, *seg, 0.0, 0, None, 0, *new.key_splits(b, H, R)), 3)
+            pair("latent_" + label, t_lat, t_old, (nseq * e * R * (p0 + n) + T * e * H * 2 * R, kvb), (2.0 * pairs * H * 2 * R, fl))
+        T = 2048
+        S = z["streams"]
+        x, xs, y = torch.randn(T, W, device=dev), torch.randn(T, S, W, device=dev), torch.randn(T, W, device=dev)
+        wv, mix, wo, wi = torch.randn(W, device=dev), torch.randn(S, S, device=dev), torch.randn(S, device=dev), torch.randn(S, device=dev)
+        ob, o32 = torch.empty(T, W, dtype=torch.bfloat16, device=dev), torch.empty(T, W, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_hyper_step", xs, y, mix, wo, wi, wv, ob, None, T, S, W, 1e-6, 1, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_rmsnorm", x, W, wv, ob, None, None, T, W, 1, 1e-6, 1, 1, None, 0, 0), 10)
+        pair("streams_write_read_norm_vs_norm_2048_rows", t_new, t_old, (T * W * (8 * S + 4 + 2), T * W * (4 + 2)))
+        # recurrences: 2048-token prompt and a decode step of 8 sequences
+        for label, ents in (("prompt_2048", [(0, 2048, 0)]), ("decode_batch8", [(600, 1, q) for q in range(8)])):
+            b = RaggedBatch.build([{"tokens": [0] * n, "pos0": p0, "slot": sl, "blocks": list(range(1, 2 + (p0 + n) // bs)), "want": []} for p0, n, sl in ents], bs, dev)
+            T = b.rows
+            ld = rh * rv + 2 * rh * rd + rh * rv
+            u = torch.randn(T, ld, device=dev) * 0.1
+            yy = torch.empty(T, rh * rv, device=dev)
+            steps = torch.empty(T, rh, 2, device=dev)
+            carry, dk = torch.empty(b.segments, rh, rd, rv, device=dev), torch.empty(b.segments, rh, device=dev)
+            t_new = timed(lambda: _call("mrs_hyb_decay_scan", u, ld, retn.decay, retn.state, yy, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, steps, carry, dk,
+                                        T, b.entries, b.segments, rh, rv, rd, rh), 5)
+            ms = ossm.s
+            uo = torch.randn(T, 2 * ms.inner + 2 * ms.groups * ms.state + ms.heads, device=dev) * 0.1
+            xbc = torch.randn(T, ms.conv_channels, device=dev) * 0.1
+            t_old = timed(lambda: _call("mrs_hyb_ssd_scan", xbc, uo, ossm.dt_bias, ossm.A_log, ossm.D, ossm.ssm_state, yy, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len,
+                                        b.ent_seg0, steps, carry, dk, T, b.entries, b.segments, ms.conv_channels, uo.stride(0), ms.inner + ms.conv_channels, ms.heads, ms.vdim, ms.state,
+                                        ms.groups), 5)
+            fl = 4.0 * T * rh * rd * rv * (3 if T > b.entries else 1)      # state update + read-out; portions run the local pass, the carry and the output pass
+            nbytes = T * 4 * (2 * rh * rv + 2 * rh * rd) + len(ents) * 8 * rh * rd * rv
+            pair("recurrence_" + label, t_new, t_old, (nbytes, nbytes), (fl, fl))
+        # per-head products in one launch against one dense product of equal work
+        T = 2048
+        qh = torch.randn(T, H * D, device=dev).to(torch.bfloat16)
+        wh = torch.randn(H, R, D, device=dev).to(torch.bfloat16)
+        wd = torch.randn(R, H * D, device=dev).to(torch.bfloat16)
+        oh = torch.empty(T, H * R, dtype=torch.bfloat16, device=dev)
+        od = torch.empty(T * H, R, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_gemm_batched", qh, wh, oh, T, R, D, H * D, D, H * R, 1, H, D, R * D, R, 1), 5)
+        t_old = timed(lambda: _call("mrs_hyb_gemm", qh, wd, od, T * H, R, D, D, H * D, R, 1, 0, None, 0, 0, 0), 5)
+        fl = 2.0 * T * H * R * D
+        pair("per_head_products_vs_dense_product_2048_rows", t_new, t_old, None, (fl, fl))
+        # projections into pages: norm + page write of the latent row / convolution of q k v against norm + rotary + page write
+        b = RaggedBatch.build([{"tokens": [0] * T, "pos0": 0, "slot": 0, "blocks": list(range(1, 2 + T // bs)), "want": []}], bs, dev)
+        ul = torch.randn(T, H * D + R, device=dev)
+        ql = torch.empty(T, H * D, dtype=torch.bfloat16, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_latent_norm_cache", ul, H * D + R, H * D, R, latent.c_norm, b.slot_mapping, ql, latent.c_cache, 1e-6, T, 1), 10)
+        nqkv = H * D + G * D + G * Dv
+        uq = torch.randn(T, nqkv, device=dev)
+        t_old = timed(lambda: _call("mrs_hyb_qk_norm_rope_cache", uq, nqkv, oattn.q_norm, oattn.k_norm, oattn.freq, b.tok_pos, b.slot_mapping, ql, oattn.k_cache, oattn.v_cache, T, H, G, D,
+                                    Dv, D // 2, bs, 1e-6, 1), 10)
+        pair("latent_norm_page_write_vs_norm_rotary_page_write", t_new, t_old, (T * (H * D + R) * (4 + 2), T * nqkv * (4 + 2)))
+        us = torch.randn(T, nqkv + H * Dv, device=dev)
+        t_c = timed(lambda: _call("mrs_hyb_conv_qkv_cache", us, us.stride(0), sink.bias, sink.conv_w, sink.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, b.tok_pos,
+                                  b.slot_mapping, ql, sink.k_cache, sink.v_cache, T, 1, H, G, D, Dv, bs, z["conv"], 0.25, 256, 1), 10)
+        pair("conv_temperature_page_write_vs_norm_rotary_page_write", t_c, t_old, (T * nqkv * (4 + 2), T * nqkv * (4 + 2)), launches=2)
+        ur = torch.randn(T, 2 * rh * rv + 2 * rh * rd, device=dev)
+        t_r = timed(lambda: _call("mrs_hyb_rotary_half", ur, ur.stride(0), rh * rv + rh * rd, rh * rv, rh, rd, rd, retn.freq, b.tok_pos, retn.k_mult, T), 10)
+        pair("half_rotary_in_place_vs_norm_rotary_page_write", t_r, t_old, (T * 2 * rh * rd * 8, T * nqkv * (4 + 2)))
+    d1 = out["models"]["setopel"]["decode"]["batch1"]
+    print(json.dumps({"metric": "setopel_decode_tokens_per_sec", "value": d1["tokens_per_sec"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": d1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"model": f"setopel-{a.setopel}", "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "setopel": out}), flush=True)
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -876,7 +1069,17 @@ def main():
     ap.add_argument("--sobunex", choices=sorted(SOBUNEX_SIZES), default=None,
                     help="instead of the default workload: a Sobunex layer list (sigmoid attention with mixed head scores, dense / routed feed-forwards; bf16) of the given size beside "
                          "a windowed-attention + routed-experts list of the package at equal size, and the like kernels of the two one by one")
+    ap.add_argument("--setopel", choices=sorted(SETOPEL_SIZES), default=None,
+                    help="instead of the default workload: a Setopel layer list (residual streams; latent / sink attention, retention; SiLU-GLU feed-forwards; bf16) of the given size "
+                         "beside an attention + state-space list of the package at equal size, and the like kernels of the two one by one")
     a = ap.parse_args()
+    if a.setopel:
+        import torch
+        dev = torch.device("cuda", 0)
+        torch.cuda.set_device(dev)
+        if a.steps == 256:
+            a.steps = 128
+        return setopel_leg(a, dev)
     if a.sobunex:
         import torch
         dev = torch.device("cuda", 0)

@@ -75,9 +75,41 @@ template <class T> __global__ void __launch_bounds__(256) rmsnorm_kernel(const f
 // u [rows, ldu] (the channels start at column 0 of the pointer handed in), cw [C, taps] (the last column multiplies the current token), state [slots, C, taps - 1]
 // (oldest first).  An entry that starts at position 0 reads zeros instead of its slot.  in_bias (nullable, [C]): the bias of the product that made u -- the convolution
 // runs over u + in_bias, and that is what the slot carries.  cb (nullable): the convolution's own bias.  act 1: SiLU of the result, 0: the result as it is.
-__global__ void __launch_bounds__(256) conv_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw, const float *__restrict__ cb,
+// Where a convolved q | k | v channel goes when the convolution feeds attention directly (ROUTE): query channels times the query temperature
+// 1 + coef ln(floor((pos + 1) / every) + 1) to q_out (T), key and value channels into the row's page slot (k_cache null: the rows carry queries only).
+struct QkvRoute {
+  void *q_out, *k_cache, *v_cache;
+  const int *tok_pos;
+  const long long *slot_mapping;
+  int nq, nk, G, D, Dv, block_size, temp_every;
+  float temp_coef;
+};
+template <class T> __device__ __forceinline__ void qkv_route(const QkvRoute &o, int t, int c, float v) {
+  if (c < o.nq) {
+    float f = 1.0f;
+    if (o.temp_every > 0) f = 1.0f + o.temp_coef * logf((float)((o.tok_pos[t] + 1) / o.temp_every + 1));
+    ((T *)o.q_out)[(size_t)t * o.nq + c] = from_f<T>(v * f);
+    return;
+  }
+  if (!o.k_cache) return;
+  const long long slot = o.slot_mapping[t];
+  if (slot < 0) return;
+  const long long blk = slot / o.block_size;
+  const int off = (int)(slot % o.block_size);
+  c -= o.nq;
+  if (c < o.nk) {
+    const int g = c / o.D, d = c % o.D;
+    ((T *)o.k_cache)[(((size_t)blk * o.G + g) * o.block_size + off) * o.D + d] = from_f<T>(v);
+  } else {
+    c -= o.nk;
+    const int g = c / o.Dv, d = c % o.Dv;
+    ((T *)o.v_cache)[(((size_t)blk * o.G + g) * o.block_size + off) * o.Dv + d] = from_f<T>(v);
+  }
+}
+template <class T, bool ROUTE> __global__ void __launch_bounds__(256) conv_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw,
+                                                   const float *__restrict__ cb,
                                                    const float *__restrict__ state, const int *__restrict__ tok_seq, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
-                                                   const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps, int act) {
+                                                   const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps, int act, QkvRoute o) {
   const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int s = tok_seq[t], r0 = seq_start[s], i = t - r0;
@@ -92,12 +124,14 @@ __global__ void __launch_bounds__(256) conv_kernel(const float *__restrict__ u, 
     else if (carried) v = st[(taps - 1) + idx];
     acc = fmaf(cw[(size_t)c * taps + j], v, acc);
   }
-  out[(size_t)t * C + c] = act ? silu_f(acc) : acc;
+  if (ROUTE) qkv_route<T>(o, t, c, acc);
+  else out[(size_t)t * C + c] = act ? silu_f(acc) : acc;
 }
 // decode steps (every entry brings one row): convolution and tap shift in one launch, the thread of (entry, channel) reads its taps, then writes them
-__global__ void __launch_bounds__(256) conv_step_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw, const float *__restrict__ cb,
+template <class T, bool ROUTE> __global__ void __launch_bounds__(256) conv_step_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw,
+                                                        const float *__restrict__ cb,
                                                         float *__restrict__ state, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot,
-                                                        float *__restrict__ out, int C, int taps, int act) {
+                                                        float *__restrict__ out, int C, int taps, int act, QkvRoute o) {
   const int s = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int row = seq_start[s], keep = taps - 1;
@@ -113,7 +147,8 @@ __global__ void __launch_bounds__(256) conv_step_kernel(const float *__restrict_
     acc = fmaf(cw[(size_t)c * taps + k], v[k], acc);
   }
   acc = fmaf(cw[(size_t)c * taps + keep], cur, acc);
-  out[(size_t)row * C + c] = act ? silu_f(acc) : acc;
+  if (ROUTE) qkv_route<T>(o, row, c, acc);
+  else out[(size_t)row * C + c] = act ? silu_f(acc) : acc;
 #pragma unroll
   for (int k = 0; k < 16; ++k) {
     if (k >= keep) break;
@@ -472,6 +507,10 @@ struct AttnArgs {
   int sink;
   const float *gate;    // nullable
   int ldg;
+  // single-row steps: `splits` > 1 workgroups (grid.z) share a row's key passes; each leaves its unnormalised sum, running maximum and sum in scratch
+  // [splits, rows, H, Dv + 2] (f32) and attn_merge_kernel joins them in split order (the sink, the gate and the rounding happen there)
+  float *scratch;
+  int splits, rows;
 };
 __device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 template <class T> struct Ld;
@@ -509,12 +548,19 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
   if (w_lo < 0) w_lo = 0;
   int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;  // kept first tokens that the window does not already cover
   if (n1 < 0) n1 = 0;
-  const int total = n1 + (i - w_lo + 1);
-  float m = a.sink ? 0.f : -FLT_MAX, l = a.sink ? 1.f : 0.f, o[DVC][2];
+  int total = n1 + (i - w_lo + 1), v_begin = 0;
+  const bool split = a.splits > 1;
+  if (split) {  // this workgroup's share of the passes
+    const int per = ((total + 63) / 64 + a.splits - 1) / a.splits;
+    v_begin = blockIdx.z * per * 64;
+    const int v_end = v_begin + per * 64;
+    total = total < v_end ? total : v_end;
+  }
+  float m = (a.sink && !split) ? 0.f : -FLT_MAX, l = (a.sink && !split) ? 1.f : 0.f, o[DVC][2];
 #pragma unroll
   for (int c = 0; c < DVC; ++c) o[c][0] = o[c][1] = 0.f;
   MRS_WAVE_SYNC();
-  for (int v0 = 0; v0 < total; v0 += 64) {
+  for (int v0 = v_begin; v0 < total; v0 += 64) {
     const int vi = v0 + lane;
     float sc = -FLT_MAX;
     long long base = -1;
@@ -538,7 +584,7 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
     }
     const float mn = fmaxf(m, wave_max(sc));
     const float alpha = expf(m - mn);
-    const float p = vi < total ? expf(sc - mn) : 0.f;
+    const float p = vi < total ? expf(sc - mn) : 0.f;  // (a split whose share is empty never gets here)
     l = l * alpha + wave_sum(p);
     m = mn;
     MRS_WAVE_SYNC();
@@ -572,6 +618,17 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
       o[c][0] = a0; o[c][1] = a1;
     }
   }
+  if (split) {
+    float *part = a.scratch + (((size_t)blockIdx.z * a.rows + t) * a.H + h) * (a.Dv + 2);
+#pragma unroll
+    for (int c = 0; c < DVC; ++c) {
+      const int d = 128 * c + 2 * lane;
+      if (d < a.Dv) part[d] = o[c][0];
+      if (d + 1 < a.Dv) part[d + 1] = o[c][1];
+    }
+    if (lane == 0) { part[a.Dv] = m; part[a.Dv + 1] = l; }
+    return;
+  }
   const float inv = 1.0f / l;
   T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
   const float *gr = a.gate ? a.gate + (size_t)t * a.ldg + (size_t)h * a.Dv : nullptr;
@@ -580,6 +637,24 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
     const int d = 128 * c + 2 * lane;
     if (d < a.Dv) out[d] = from_f<T>(o[c][0] * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
     if (d + 1 < a.Dv) out[d + 1] = from_f<T>(o[c][1] * inv * (gr ? sigmoid_f(gr[d + 1]) : 1.0f));
+  }
+}
+// joins the splits of a row and head: M = max_s m_s (and 0 with the sink), L = sum_s l_s e^{m_s - M} (+ e^{-M}), out = sum_s o_s e^{m_s - M} / L (times sigmoid(gate))
+template <class T> __global__ void __launch_bounds__(64) attn_merge_kernel(AttnArgs a) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, stride = a.Dv + 2;
+  const float *base = a.scratch + ((size_t)t * a.H + h) * stride;
+  const size_t step = (size_t)a.rows * a.H * stride;
+  float M = a.sink ? 0.f : -FLT_MAX;
+  for (int s = 0; s < a.splits; ++s) M = fmaxf(M, base[s * step + a.Dv]);
+  float L = a.sink ? expf(-M) : 0.f;
+  for (int s = 0; s < a.splits; ++s) L += base[s * step + a.Dv + 1] * expf(base[s * step + a.Dv] - M);
+  const float inv = 1.0f / L;
+  T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
+  const float *gr = a.gate ? a.gate + (size_t)t * a.ldg + (size_t)h * a.Dv : nullptr;
+  for (int d = lane; d < a.Dv; d += 64) {
+    float acc = 0.f;
+    for (int s = 0; s < a.splits; ++s) acc = fmaf(base[s * step + d], expf(base[s * step + a.Dv] - M), acc);
+    out[d] = from_f<T>(acc * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
   }
 }
 
@@ -1066,19 +1141,40 @@ extern "C" int mrs_hyb_rmsnorm(const float *x, int ldx, const float *w, void *ou
   return ok_or("mrs_hyb_rmsnorm");
 }
 
-/* out [rows, C] = act(conv(u + in_bias) + cb): in_bias, cb nullable; act 1 = SiLU, 0 = none.  The slots carry the last taps - 1 rows of u + in_bias. */
-extern "C" int mrs_hyb_conv(const float *u, int ldu, const float *in_bias, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start,
-                            const int *seq_pos0, const int *seq_slot, float *out, int rows, int entries, int C, int taps, int act, void *stream) {
+/* out [rows, C] = act(conv(u + in_bias) + cb): in_bias, cb nullable; act 1 = SiLU, 0 = none.  The slots carry the last taps - 1 rows of u + in_bias.  With a route (dtype
+ * 1 | 2) the result goes to the query buffer / the K and V pages instead of `out`. */
+static int conv_launch(const float *u, int ldu, const float *in_bias, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start,
+                       const int *seq_pos0, const int *seq_slot, float *out, int rows, int entries, int C, int taps, int act, const QkvRoute &o, int dtype, void *stream) {
   if (rows <= 0) return 0;
   if (taps < 1 || taps > 17) return fail("mrs_hyb_conv: 1 .. 17 taps");
-  if (rows == entries) {  // one row per entry (an entry without rows cannot occur then)
-    hipLaunchKernelGGL(conv_step_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, seq_start, seq_pos0, seq_slot, out, C, taps, act);
-    return ok_or("mrs_hyb_conv");
-  }
-  hipLaunchKernelGGL(conv_kernel, dim3(rows, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps, act);
-  if (taps > 1)
-    hipLaunchKernelGGL(conv_state_kernel, dim3(entries, (C + 255) / 256), dim3(256), 0, S_(stream), u, ldu, in_bias, state, seq_start, seq_pos0, seq_slot, C, taps);
+  if (taps > 1 && !state) return fail("mrs_hyb_conv: carried taps need their slots");
+  dim3 g_rows(rows, (C + 255) / 256), g_ent(entries, (C + 255) / 256);
+  const bool step = rows == entries;  // one row per entry (an entry without rows cannot occur then)
+#define MRS_CONV(T, R) do { if (step) hipLaunchKernelGGL((conv_step_kernel<T, R>), g_ent, dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, seq_start, seq_pos0, seq_slot, out, C, taps, act, o); \
+                            else hipLaunchKernelGGL((conv_kernel<T, R>), g_rows, dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps, act, o); } while (0)
+  if (dtype == 0) MRS_CONV(float, false);
+  else if (dtype == 1) MRS_CONV(mrs::bf16_t, true);
+  else if (dtype == 2) MRS_CONV(float, true);
+  else return fail("mrs_hyb_conv: dtype");
+#undef MRS_CONV
+  if (!step && taps > 1)
+    hipLaunchKernelGGL(conv_state_kernel, g_ent, dim3(256), 0, S_(stream), u, ldu, in_bias, state, seq_start, seq_pos0, seq_slot, C, taps);
   return ok_or("mrs_hyb_conv");
+}
+extern "C" int mrs_hyb_conv(const float *u, int ldu, const float *in_bias, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start,
+                            const int *seq_pos0, const int *seq_slot, float *out, int rows, int entries, int C, int taps, int act, void *stream) {
+  return conv_launch(u, ldu, in_bias, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, rows, entries, C, taps, act, QkvRoute{}, 0, stream);
+}
+/* The convolution over the q | k | v columns of u (+ in_bias, no activation) feeding attention in the same launch: q times the query temperature (temp_every <= 0: none) to
+ * q_out (dtype), k and v into the rows' page slots.  k_cache null: u carries H * D query columns only. */
+extern "C" int mrs_hyb_conv_qkv_cache(const float *u, int ldu, const float *in_bias, const float *cw, float *state, const int *tok_seq, const int *seq_start, const int *seq_pos0,
+                                      const int *seq_slot, const int *tok_pos, const long long *slot_mapping, void *q_out, void *k_cache, void *v_cache, int rows, int entries, int H,
+                                      int G, int D, int Dv, int block_size, int taps, float temp_coef, int temp_every, int dtype, void *stream) {
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || (k_cache && !v_cache) || !q_out) return fail("mrs_hyb_conv_qkv_cache: head sizes (heads % kv_heads == 0)");
+  if (dtype != 1 && dtype != 2) return fail("mrs_hyb_conv_qkv_cache: dtype");
+  const QkvRoute o{q_out, k_cache, v_cache, tok_pos, slot_mapping, H * D, G * D, G, D, Dv, block_size, temp_every, temp_coef};
+  const int C = H * D + (k_cache ? G * D + G * Dv : 0);
+  return conv_launch(u, ldu, in_bias, cw, nullptr, state, tok_seq, seq_start, seq_pos0, seq_slot, nullptr, rows, entries, C, taps, 0, o, dtype, stream);
 }
 extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const float *cb, float *state, const int *tok_seq, const int *seq_start, const int *seq_pos0,
                                  const int *seq_slot, float *out, int rows, int entries, int C, int taps, void *stream) {
@@ -1164,11 +1260,12 @@ extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float 
  * query-tiled kernel */
 static int attn_launch(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
                        int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
-                       const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg, void *stream) {
+                       const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg,
+                       float *scratch, int splits, void *stream) {
   if (rows <= 0) return 0;
   if (Dv > 512 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 512 / heads % kv_heads");
   if (gate && ldg < H * Dv) return fail("mrs_hyb_paged_window_attn: gate rows shorter than heads * value size");
-  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg};
+  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg, nullptr, 0, rows};
   const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
   const int c = (Dv + 127) / 128;
   if (vec && seg_entry && segments > 0 && rows > segments && segments <= 65535 && seg_rows > 0) {
@@ -1185,13 +1282,22 @@ static int attn_launch(const void *q, const void *k_cache, const void *v_cache, 
     }
   }
   const size_t lds = (size_t)(((D + 3) & ~3) + 64) * 4 + 64 * 8;
-  dim3 grid(rows, H);
+  if (scratch && splits > 1) {
+    if (splits > 256) return fail("mrs_hyb_paged_window_attn: more than 256 key splits");
+    a.scratch = scratch;
+    a.splits = splits;
+  }
+  dim3 grid(rows, H, a.splits > 1 ? a.splits : 1);
 #define MRS_ATTN(T, C) do { if (vec) hipLaunchKernelGGL((paged_window_attn_kernel<T, C, true>), grid, dim3(64), lds, S_(stream), a); \
                             else hipLaunchKernelGGL((paged_window_attn_kernel<T, C, false>), grid, dim3(64), lds, S_(stream), a); } while (0)
   if (dtype == 1) { if (c <= 1) MRS_ATTN(mrs::bf16_t, 1); else if (c <= 2) MRS_ATTN(mrs::bf16_t, 2); else MRS_ATTN(mrs::bf16_t, 4); }
   else if (dtype == 2) { if (c <= 1) MRS_ATTN(float, 1); else if (c <= 2) MRS_ATTN(float, 2); else MRS_ATTN(float, 4); }
   else return fail("mrs_hyb_paged_window_attn: dtype");
 #undef MRS_ATTN
+  if (a.splits > 1) {
+    if (dtype == 1) hipLaunchKernelGGL(attn_merge_kernel<mrs::bf16_t>, dim3(rows, H), dim3(64), 0, S_(stream), a);
+    else hipLaunchKernelGGL(attn_merge_kernel<float>, dim3(rows, H), dim3(64), 0, S_(stream), a);
+  }
   return ok_or("mrs_hyb_paged_window_attn");
 }
 
@@ -1199,15 +1305,16 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
                                          int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
                                          const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream) {
   return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, dtype, seg_entry, seg_row0, seg_len,
-                     segments, seg_rows, 0.f, 0, nullptr, 0, stream);
+                     segments, seg_rows, 0.f, 0, nullptr, 0, nullptr, 0, stream);
 }
-/* the same attention with its options: softcap (0: none), sink (a zero-score term in the denominator), gate (nullable f32 [rows, ldg]: output times sigmoid(gate)) */
+/* the same attention with its options: softcap (0: none), sink (a zero-score term in the denominator), gate (nullable f32 [rows, ldg]: output times sigmoid(gate)).
+ * scratch (nullable, f32 [splits, rows, H, Dv + 2]) with splits > 1: a step of single rows deals every row's key passes to that many workgroups (steps with portions ignore it) */
 extern "C" int mrs_hyb_paged_attn_opts(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
                                        int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
                                        const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg,
-                                       void *stream) {
+                                       float *scratch, int splits, void *stream) {
   return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, dtype, seg_entry, seg_row0, seg_len,
-                     segments, seg_rows, softcap, sink, gate, ldg, stream);
+                     segments, seg_rows, softcap, sink, gate, ldg, scratch, splits, stream);
 }
 
 /* h [rows, W] f32 (contiguous), wr [E (+ 1), W] f32 */

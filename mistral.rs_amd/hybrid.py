@@ -34,8 +34,9 @@ _SIGS = {
     "mrs_hyb_embed": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "mrs_hyb_rmsnorm": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _f, _i, _i, _vp, _i, _i, _vp],
     "mrs_hyb_conv": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "mrs_hyb_conv_qkv_cache": [_vp, _i] + [_vp] * 12 + [_i] * 8 + [_f, _i, _i, _vp],
     "mrs_hyb_decay_scan": [_vp, _i] + [_vp] * 12 + [_i] * 7 + [_vp],
-    "mrs_hyb_paged_attn_opts": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _i, _vp],
+    "mrs_hyb_paged_attn_opts": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _i, _vp, _i, _vp],
     "mrs_hyb_rotary_half": [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _f, _i, _vp],
     "mrs_hyb_latent_norm_cache": [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _i, _vp],
     "mrs_hyb_hyper_step": [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _vp],
@@ -801,19 +802,18 @@ class GatedSinkAttention(_Module):
         u = m.linear(h, self.w_in)                                         # f32 [T, q | k | v | gate logits]
         qb = self.bias[:self.nq]
         kb, vb = (self.bias[self.nq:self.nq + self.nk], self.bias[self.nq + self.nk:]) if self.own else (None, None)
-        src_rows, ld = u, u.stride(0)
-        if s.conv:
-            src_rows = torch.empty(T, self.channels, dtype=torch.float32, device=m.device)
-            _call("mrs_hyb_conv", u, u.stride(0), self.bias, self.conv_w, None, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, src_rows, T, b.entries,
-                  self.channels, s.conv, 0)
-            ld, qb, kb, vb = self.channels, None, None, None
         q = torch.empty(T, self.nq, dtype=m.torch_dtype, device=m.device)
-        _call("mrs_hyb_qkv_bias_temp_cache", src_rows, ld, qb, kb, vb, b.tok_pos, b.slot_mapping, q, self.k_cache, self.v_cache, T, s.heads, s.kv_heads, s.dim, s.vdim,
-              m.block_size, s.temp_coef, s.temp_every, m.dt)
+        if s.conv:   # bias, convolution, temperature and the page write in one launch (the slots' taps in a second one when a portion is in the batch)
+            _call("mrs_hyb_conv_qkv_cache", u, u.stride(0), self.bias, self.conv_w, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, b.tok_pos, b.slot_mapping, q,
+                  self.k_cache, self.v_cache, T, b.entries, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, s.conv, s.temp_coef, s.temp_every, m.dt)
+        else:
+            _call("mrs_hyb_qkv_bias_temp_cache", u, u.stride(0), qb, kb, vb, b.tok_pos, b.slot_mapping, q, self.k_cache, self.v_cache, T, s.heads, s.kv_heads, s.dim, s.vdim,
+                  m.block_size, s.temp_coef, s.temp_every, m.dt)
         src = self if self.own else m.layers[s.kv_from].mixer               # that layer ran earlier in this step: its pages hold this step's rows already
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
         _call("mrs_hyb_paged_attn_opts", q, src.k_cache, src.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, b.max_blocks,
-              0, 0, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, s.softcap, int(s.sink), u[:, self.gate_col:], u.stride(0))
+              0, 0, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, s.softcap, int(s.sink), u[:, self.gate_col:], u.stride(0),
+              *m.key_splits(b, s.heads, s.vdim))
         m.linear(o, self.w_o, out=x, accumulate=accumulate)
 
 
@@ -909,7 +909,7 @@ class LatentAttention(_Module):
         qa = m.batched_linear(q, self.w_ukT, H)                            # [T, H * kv_rank] in the serving dtype
         oa = torch.empty(T, H * R, dtype=dt, device=dev)
         _call("mrs_hyb_paged_attn_opts", qa, self.c_cache, self.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, m.block_size, b.max_blocks, 0, 0, s.scale,
-              m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, 0, None, 0)
+              m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, 0, None, 0, *m.key_splits(b, H, R))
         ov = m.batched_linear(oa, self.w_uv, H)                            # [T, H * vdim]
         m.linear(ov, self.w_o, out=x, accumulate=accumulate)
 
@@ -1048,6 +1048,20 @@ class HybridDecoder:
         if norm_w is None:
             return out32
         return (out, out32) if want32 else out
+
+    KEY_SPLIT_ROWS = 128   # steps of single rows up to this many rows split their keys
+    KEYS_PER_SPLIT = 256   # at least this many keys (of the longest table in the batch) per workgroup
+    KEY_SPLITS = 32
+
+    def key_splits(self, b: RaggedBatch, heads: int, vdim: int):
+        """(scratch, splits) for an attention launch over unwindowed keys: a step in which every entry brings one row deals each row's keys to several workgroups
+        (one wave walking thousands of keys is latency-bound); (None, 0) otherwise."""
+        if b.seg_rows != 1 or b.rows > self.KEY_SPLIT_ROWS:
+            return None, 0
+        splits = min(self.KEY_SPLITS, (b.max_blocks * self.block_size) // self.KEYS_PER_SPLIT)
+        if splits < 2:
+            return None, 0
+        return torch.empty(splits, b.rows, heads, vdim + 2, dtype=torch.float32, device=self.device), splits
 
     def batched_linear(self, a, w, heads: int):
         """a [M, heads * K] (column block h = the operand of head h), w [heads, N, K] -> [M, heads * N] in the serving dtype, rounded once: per-head products whose

@@ -477,7 +477,7 @@ def test_planted_keys_sink_and_cap(dev, dtype):
     att.v_cache[blk, :, off] = v.to(dev, td)
     tol = 1e-4 if dtype == "float32" else 2e-2
 
-    def run(i, k, q, rows, cap=0.0, sink=1, gate=None):
+    def run(i, k, q, rows, cap=0.0, sink=1, gate=None, splits=0):
         att.k_cache[blk, :, off] = k.to(dev, td)
         p0 = i if rows == "decode" else max(0, i - 20)
         n = i - p0 + 1
@@ -485,9 +485,13 @@ def test_planted_keys_sink_and_cap(dev, dtype):
         qq = torch.zeros(n, H * D, dtype=td, device=dev)
         qq[n - 1] = q.reshape(-1).to(dev, td)
         out = torch.empty(n, H * Dv, dtype=td, device=dev)
+        if rows == "decode" and not splits:
+            splits = 1 + (i + j0) % 6                         # the keys dealt to several workgroups (some of them without a share), or all to one
+        scratch = torch.full((max(splits, 1), n, H, Dv + 2), float("nan"), device=dev) if splits > 1 else None
         _call("mrs_hyb_paged_attn_opts", qq, att.k_cache, att.v_cache, b.block_tables, b.tok_seq, b.tok_pos, out, n, H, G, D, Dv, bs, b.max_blocks, 0, 0, 1.0, m.dt,
-              b.seg_entry, b.seg_row0, b.seg_len, b.segments, 64, cap, sink, gate, H * Dv if gate is not None else 0)
+              b.seg_entry, b.seg_row0, b.seg_len, b.segments, 64, cap, sink, gate, H * Dv if gate is not None else 0, scratch, splits if splits > 1 else 0)
         return out[n - 1].double().cpu().view(H, Dv)
+    j0 = 0
     for i in (60, 64, 95, 96, 299):
         for j in (0, i, 31, 32, i - 1, i - 63, i - 64, i - 65, i + 1, 3):
             if j < 0 or j >= T:
@@ -496,6 +500,7 @@ def test_planted_keys_sink_and_cap(dev, dtype):
             k[j, 0, 0] = 6.0
             q = torch.zeros(H, D, dtype=torch.bfloat16)
             q[1, 0] = 6.0                                    # head 1 asks for key j; head 0 asks for nothing and averages what it sees with the sink
+            j0 = j
             for rows in ("decode", "prompt"):
                 got = run(i, k, q, rows)
                 if j <= i:
@@ -525,6 +530,28 @@ def test_planted_keys_sink_and_cap(dev, dtype):
         got = run(100, k, q, rows, cap=2.0, gate=gd.to(dev))
         assert float((got[0] - want * torch.sigmoid(gate[0, :Dv].double())).abs().max()) < tol
     sv.end(1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,bar", [("float32", 3e-5), ("bfloat16", 4e-2)])
+def test_decoding_with_the_keys_dealt_to_several_workgroups(dev, dtype, bar, monkeypatch):
+    """single-row steps over a few hundred keys with a small share per workgroup: three sequences of unequal length in one step (the shortest leaves most workgroups without
+    keys), against the restatement; and the same step without the split"""
+    from mistralrs_amd.hybrid import HybridDecoder
+    cfg = config([attn(), lat(), attn(kv_from=0, conv=0), lat(heads=2, dim=8, vdim=8, rank=136, mlp=None)])
+    w = weights(cfg, 31)
+    wd = f64(w)
+    req = {1: toks(330, cfg["vocab"], 81), 2: toks(70, cfg["vocab"], 82), 3: toks(9, cfg["vocab"], 83)}
+    full = {r: O.forward(cfg, wd, t) for r, t in req.items()}
+    for per in (64, 10 ** 9):
+        monkeypatch.setattr(HybridDecoder, "KEYS_PER_SPLIT", per)
+        sv = Served(cfg, w, dev, dtype, max_tokens=512)
+        sv.step([(r, t[:-8]) for r, t in req.items()])
+        assert (sv.m.key_splits(_batch(dev, [(320, 1, 0)]), 4, 8)[1] > 1) == (per == 64)
+        for i in range(8):
+            outs = sv.step([(r, [t[len(t) - 8 + i]]) for r, t in req.items()])
+            for (r, t), o in zip(req.items(), outs):
+                assert close(o, full[r][len(t) - 8 + i:len(t) - 7 + i], bar), (per, r, i)
 
 
 @pytest.mark.gpu
