@@ -106,26 +106,52 @@ template <class T> __device__ __forceinline__ void qkv_route(const QkvRoute &o, 
     ((T *)o.v_cache)[(((size_t)blk * o.G + g) * o.block_size + off) * o.Dv + d] = from_f<T>(v);
   }
 }
+// A thread owns one channel of CONV_ROWS consecutive rows and slides a register window of the last taps - 1 inputs along them (every input is loaded once, the taps' weights
+// once); the window is filled afresh at the block's first row and wherever a new entry starts.  Taps in ascending order, as the step kernel adds them.
+constexpr int CONV_ROWS = 8;
 template <class T, bool ROUTE> __global__ void __launch_bounds__(256) conv_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw,
                                                    const float *__restrict__ cb,
                                                    const float *__restrict__ state, const int *__restrict__ tok_seq, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
-                                                   const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps, int act, QkvRoute o) {
-  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+                                                   const int *__restrict__ seq_slot, float *__restrict__ out, int C, int taps, int act, QkvRoute o, int rows) {
+  const int t0 = blockIdx.x * CONV_ROWS, c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
-  const int s = tok_seq[t], r0 = seq_start[s], i = t - r0;
-  const bool carried = seq_pos0[s] > 0;
-  const float *st = state + ((size_t)seq_slot[s] * C + c) * (taps - 1);
-  const float ib = in_bias ? in_bias[c] : 0.f;
-  float acc = cb ? cb[c] : 0.f;
-  for (int j = 0; j < taps; ++j) {
-    const int idx = i - (taps - 1) + j;
-    float v = 0.f;
-    if (idx >= 0) v = u[(size_t)(r0 + idx) * ldu + c] + ib;
-    else if (carried) v = st[(taps - 1) + idx];
-    acc = fmaf(cw[(size_t)c * taps + j], v, acc);
+  const int keep = taps - 1;
+  const float ib = in_bias ? in_bias[c] : 0.f, b0 = cb ? cb[c] : 0.f;
+  float w[16], win[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) w[k] = k < keep ? cw[(size_t)c * taps + k] : 0.f;
+  const float w_cur = cw[(size_t)c * taps + keep];
+#pragma unroll
+  for (int r = 0; r < CONV_ROWS; ++r) {
+    const int t = t0 + r;
+    if (t >= rows) break;
+    const int s = tok_seq[t], r0 = seq_start[s], i = t - r0;
+    if (r == 0 || i == 0) {
+      const bool carried = seq_pos0[s] > 0;
+      const float *st = state + ((size_t)seq_slot[s] * C + c) * keep;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        if (k >= keep) break;
+        const int idx = i - keep + k;
+        win[k] = idx >= 0 ? u[(size_t)(r0 + idx) * ldu + c] + ib : (carried ? st[keep + idx] : 0.f);
+      }
+    }
+    const float cur = u[(size_t)t * ldu + c] + ib;
+    float acc = b0;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      if (k >= keep) break;
+      acc = fmaf(w[k], win[k], acc);
+    }
+    acc = fmaf(w_cur, cur, acc);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      if (k >= keep) break;
+      win[k] = k + 1 < keep ? win[k + 1] : cur;
+    }
+    if (ROUTE) qkv_route<T>(o, t, c, acc);
+    else out[(size_t)t * C + c] = act ? silu_f(acc) : acc;
   }
-  if (ROUTE) qkv_route<T>(o, t, c, acc);
-  else out[(size_t)t * C + c] = act ? silu_f(acc) : acc;
 }
 // decode steps (every entry brings one row): convolution and tap shift in one launch, the thread of (entry, channel) reads its taps, then writes them
 template <class T, bool ROUTE> __global__ void __launch_bounds__(256) conv_step_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ in_bias, const float *__restrict__ cw,
@@ -1148,10 +1174,10 @@ static int conv_launch(const float *u, int ldu, const float *in_bias, const floa
   if (rows <= 0) return 0;
   if (taps < 1 || taps > 17) return fail("mrs_hyb_conv: 1 .. 17 taps");
   if (taps > 1 && !state) return fail("mrs_hyb_conv: carried taps need their slots");
-  dim3 g_rows(rows, (C + 255) / 256), g_ent(entries, (C + 255) / 256);
+  dim3 g_rows((rows + CONV_ROWS - 1) / CONV_ROWS, (C + 255) / 256), g_ent(entries, (C + 255) / 256);
   const bool step = rows == entries;  // one row per entry (an entry without rows cannot occur then)
 #define MRS_CONV(T, R) do { if (step) hipLaunchKernelGGL((conv_step_kernel<T, R>), g_ent, dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, seq_start, seq_pos0, seq_slot, out, C, taps, act, o); \
-                            else hipLaunchKernelGGL((conv_kernel<T, R>), g_rows, dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps, act, o); } while (0)
+                            else hipLaunchKernelGGL((conv_kernel<T, R>), g_rows, dim3(256), 0, S_(stream), u, ldu, in_bias, cw, cb, state, tok_seq, seq_start, seq_pos0, seq_slot, out, C, taps, act, o, rows); } while (0)
   if (dtype == 0) MRS_CONV(float, false);
   else if (dtype == 1) MRS_CONV(mrs::bf16_t, true);
   else if (dtype == 2) MRS_CONV(float, true);
