@@ -965,19 +965,33 @@ def setopel_leg(a, dev):
             o = torch.empty(T, H * Dv, dtype=torch.bfloat16, device=dev)
             seg = (b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
             t_new = timed(lambda: _call("mrs_hyb_paged_attn_opts", qn, sink.k_cache, sink.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, 0, 0,
-                                        D ** -0.5, 1, *seg, 30.0, 1, gate, H * Dv, *new.key_splits(b, H, Dv)), 5)
+                                        D ** -0.5, 1, *seg, 30.0, 1, gate, H * Dv, *new.key_splits(b, H, Dv), 0), 5)
             t_old = timed(lambda: _call("mrs_hyb_paged_window_attn", qn, oattn.k_cache, oattn.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, 0, 0,
                                         D ** -0.5, 1, *seg), 5)
             pairs = sum(p0 + i + 1 for i in range(n)) * nseq
             fl = 2.0 * pairs * H * (D + Dv)
             kvb = nseq * e * G * (D + Dv) * (p0 + n) + T * e * H * (D + Dv)
             pair("sink_" + label, t_new, t_old, (kvb + T * H * Dv * 4, kvb), (fl, fl))
-            # latent attention: the same kernel, one shared head of `rank` dimensions for keys and values
-            qa = torch.randn(T, H * R, device=dev).to(torch.bfloat16)
-            oa = torch.empty(T, H * R, dtype=torch.bfloat16, device=dev)
-            t_lat = timed(lambda: _call("mrs_hyb_paged_attn_opts", qa, latent.c_cache, latent.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, bs, b.max_blocks, 0, 0,
-                                        D ** -0.5, 1, *seg, 0.0, 0, None, 0, *new.key_splits(b, H, R)), 3)
-            pair("latent_" + label, t_lat, t_old, (nseq * e * R * (p0 + n) + T * e * H * 2 * R, kvb), (2.0 * pairs * H * 2 * R, fl))
+            # latent attention: single rows read the cached latent rows (one shared head of `rank` dimensions for keys and values); prompt steps gather the context's
+            # blocks, expand them into keys and values and read those
+            if n == 1:
+                qa = torch.randn(T, H * R, device=dev).to(torch.bfloat16)
+                oa = torch.empty(T, H * R, dtype=torch.bfloat16, device=dev)
+                t_lat = timed(lambda: _call("mrs_hyb_paged_attn_opts", qa, latent.c_cache, latent.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, bs, b.max_blocks, 0, 0,
+                                            D ** -0.5, 1, *seg, 0.0, 0, None, 0, *new.key_splits(b, H, R), 0), 3)
+                pair("latent_" + label, t_lat, t_old, (nseq * e * R * (p0 + n) + T * e * H * 2 * R, kvb), (2.0 * pairs * H * 2 * R, fl))
+            else:
+                assert latent.expands(b)
+                tables, source, nblk = b.context_blocks()
+
+                def expanded():
+                    c = torch.empty(nblk * bs, R, dtype=torch.bfloat16, device=dev)
+                    _call("mrs_hyb_gather_rows", latent.c_cache, source, c, nblk, bs * R * e // 4)
+                    k, v = new.linear_rounded(c, latent.w_uk), new.linear_rounded(c, latent.w_uv.view(H * Dv, R))
+                    _call("mrs_hyb_paged_attn_opts", qn, k, v, tables, b.tok_seq, b.tok_pos, o, T, H, H, D, Dv, bs, b.max_blocks, 0, 0, D ** -0.5, 1, *seg, 0.0, 0, None, 0, None, 0, 1)
+                t_lat = timed(expanded, 3)
+                fl_lat = 2.0 * pairs * H * (D + Dv) + 2.0 * nblk * bs * R * H * (D + Dv)
+                pair("latent_expanded_" + label, t_lat, t_old, (nseq * e * R * (p0 + n) + T * e * H * (D + Dv), kvb), (fl_lat, fl), launches=4)
         T = 2048
         S = z["streams"]
         x, xs, y = torch.randn(T, W, device=dev), torch.randn(T, S, W, device=dev), torch.randn(T, W, device=dev)

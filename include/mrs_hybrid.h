@@ -24,7 +24,7 @@ int mrs_hyb_conv_qkv_cache(const float *u, int ldu, const float *in_bias, const 
 int mrs_hyb_decay_scan(const float *xkq, int ld, const float *fixed_decay, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry, float *decay, int rows, int entries, int segments, int heads, int P, int N, int G, void *stream);
 int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping, void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype, void *stream);
 int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out, int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype, const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream);
-int mrs_hyb_paged_attn_opts(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out, int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype, const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg, float *scratch, int splits, void *stream);
+int mrs_hyb_paged_attn_opts(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out, int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype, const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg, float *scratch, int splits, int token_major, void *stream);
 int mrs_hyb_route_sigmoid_topk(const float *h, const float *wr, int rows, int W, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream);
 int mrs_hyb_moe_dispatch(const int *ids, int R, int E, int *bounds, int *sorted_route, int *route_pos, int *sorted_expert, void *stream);
 int mrs_hyb_moe_gather(const float *h32, const int *sorted_route, const float *wts, int top, void *out, int R, int W, int dtype, void *stream);

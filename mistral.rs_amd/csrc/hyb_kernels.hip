@@ -537,7 +537,13 @@ struct AttnArgs {
   // [splits, rows, H, Dv + 2] (f32) and attn_merge_kernel joins them in split order (the sink, the gate and the rounding happen there)
   float *scratch;
   int splits, rows;
+  int token_major;      // K / V rows laid out [block, slot, kv head, dim] (a product's row-major output) instead of [block, kv head, slot, dim]
 };
+__device__ __forceinline__ long long kv_row(const AttnArgs &a, const int *bt, int key, int g) {
+  const long long blk = bt[key / a.block_size];
+  const int off = key % a.block_size;
+  return a.token_major ? (blk * a.block_size + off) * a.G + g : (blk * a.G + g) * a.block_size + off;
+}
 __device__ __forceinline__ float capped(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 template <class T> struct Ld;
 template <> struct Ld<bf16_t> {
@@ -592,7 +598,7 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
     long long base = -1;
     if (vi < total) {
       const int key = vi < n1 ? vi : w_lo + (vi - n1);
-      base = ((long long)bt[key / a.block_size] * a.G + g) * a.block_size + key % a.block_size;
+      base = kv_row(a, bt, key, g);
       const T *kr = (const T *)a.k_cache + (size_t)base * a.D;
       float acc = 0.f;
       if (VEC) {
@@ -726,7 +732,7 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
     for (int q = 0; q < NQ; ++q) sc[q] = 0.f;
     if (vi < total) {
       key = vi < n1 ? vi : w_lo + (vi - n1);
-      base = ((long long)bt[key / a.block_size] * a.G + g) * a.block_size + key % a.block_size;
+      base = kv_row(a, bt, key, g);
       const T *kr = (const T *)a.k_cache + (size_t)base * a.D;
       for (int d = 0; d < a.D; d += 8) {
         float kv[8];
@@ -1287,11 +1293,11 @@ extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float 
 static int attn_launch(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
                        int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
                        const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg,
-                       float *scratch, int splits, void *stream) {
+                       float *scratch, int splits, int token_major, void *stream) {
   if (rows <= 0) return 0;
   if (Dv > 512 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 512 / heads % kv_heads");
   if (gate && ldg < H * Dv) return fail("mrs_hyb_paged_window_attn: gate rows shorter than heads * value size");
-  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg, nullptr, 0, rows};
+  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg, nullptr, 0, rows, token_major ? 1 : 0};
   const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
   const int c = (Dv + 127) / 128;
   if (vec && seg_entry && segments > 0 && rows > segments && segments <= 65535 && seg_rows > 0) {
@@ -1331,16 +1337,17 @@ extern "C" int mrs_hyb_paged_window_attn(const void *q, const void *k_cache, con
                                          int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
                                          const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, void *stream) {
   return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, dtype, seg_entry, seg_row0, seg_len,
-                     segments, seg_rows, 0.f, 0, nullptr, 0, nullptr, 0, stream);
+                     segments, seg_rows, 0.f, 0, nullptr, 0, nullptr, 0, 0, stream);
 }
 /* the same attention with its options: softcap (0: none), sink (a zero-score term in the denominator), gate (nullable f32 [rows, ldg]: output times sigmoid(gate)).
- * scratch (nullable, f32 [splits, rows, H, Dv + 2]) with splits > 1: a step of single rows deals every row's key passes to that many workgroups (steps with portions ignore it) */
+ * scratch (nullable, f32 [splits, rows, H, Dv + 2]) with splits > 1: a step of single rows deals every row's key passes to that many workgroups (steps with portions ignore it).
+ * token_major: k_cache / v_cache hold rows [block, slot, kv head, dim], the row-major output of a product over the blocks' tokens */
 extern "C" int mrs_hyb_paged_attn_opts(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
                                        int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
                                        const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg,
-                                       float *scratch, int splits, void *stream) {
+                                       float *scratch, int splits, int token_major, void *stream) {
   return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, dtype, seg_entry, seg_row0, seg_len,
-                     segments, seg_rows, softcap, sink, gate, ldg, scratch, splits, stream);
+                     segments, seg_rows, softcap, sink, gate, ldg, scratch, splits, token_major, stream);
 }
 
 /* h [rows, W] f32 (contiguous), wr [E (+ 1), W] f32 */

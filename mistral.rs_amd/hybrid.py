@@ -36,7 +36,7 @@ _SIGS = {
     "mrs_hyb_conv": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "mrs_hyb_conv_qkv_cache": [_vp, _i] + [_vp] * 12 + [_i] * 8 + [_f, _i, _i, _vp],
     "mrs_hyb_decay_scan": [_vp, _i] + [_vp] * 12 + [_i] * 7 + [_vp],
-    "mrs_hyb_paged_attn_opts": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _i, _vp, _i, _vp],
+    "mrs_hyb_paged_attn_opts": [_vp] * 7 + [_i] * 9 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _i, _vp, _i, _i, _vp],
     "mrs_hyb_rotary_half": [_vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _f, _i, _vp],
     "mrs_hyb_latent_norm_cache": [_vp, _i, _i, _i, _vp, _vp, _vp, _vp, _f, _i, _i, _vp],
     "mrs_hyb_hyper_step": [_vp] * 8 + [_i, _i, _i, _f, _i, _i, _vp],
@@ -101,6 +101,24 @@ class RaggedBatch:
     seg_len: Optional[torch.Tensor] = None     # i32 [segments]
     ent_seg0: Optional[torch.Tensor] = None    # i32 [entries + 1]  first segment of every entry, then the total
     seg_rows: int = 0                          # rows of the longest segment (1: every entry brings one decoded token)
+    host_blocks: Optional[List[Sequence[int]]] = None   # every entry's block ids covering its last position (host copy; `build` keeps it)
+    _context: Optional[tuple] = None
+
+    def context_blocks(self):
+        """The blocks that hold the batch's whole contexts, renumbered densely: (tables i32 [entries, max_blocks] of dense ids, source i32 [n] = the pool block behind
+        dense block d, n).  A mixer that expands its cached rows for a prompt step (keys and values from latent rows) gathers the source blocks into a scratch and reads the
+        scratch through these tables."""
+        if self._context is None:
+            if self.host_blocks is None:
+                raise ValueError("RaggedBatch: this batch was not built from entries")
+            tables = np.zeros((self.entries, self.max_blocks), dtype=np.int32)
+            src: List[int] = []
+            for s, blocks in enumerate(self.host_blocks):
+                tables[s, :len(blocks)] = np.arange(len(src), len(src) + len(blocks), dtype=np.int32)
+                src.extend(int(x) for x in blocks)
+            dev = self.tokens.device
+            self._context = (torch.from_numpy(tables).to(dev), torch.tensor(src, dtype=torch.int32, device=dev), len(src))
+        return self._context
 
     SEGMENT = int(os.environ.get("MRS_HYB_SEGMENT", "64"))   # rows per segment
 
@@ -122,6 +140,7 @@ class RaggedBatch:
             o += n
         tok, tseq, tpos, sst, sp0, ssl, bt, sge, sgr, sgl, es0 = views
         z = 0
+        host_blocks = []
         bt = bt.reshape(S, mb)
         slots = np.zeros(T, dtype=np.int64)
         want: List[int] = []
@@ -131,6 +150,7 @@ class RaggedBatch:
             blocks = np.asarray(e["blocks"], dtype=np.int64)
             if n and (p0 + n - 1) // block_size >= len(blocks):
                 raise ValueError("RaggedBatch: the entry's blocks do not cover its last position")
+            host_blocks.append(blocks[:(p0 + n - 1) // block_size + 1] if n else blocks[:0])
             tok[r:r + n] = e["tokens"]
             tseq[r:r + n] = s
             pos = np.arange(p0, p0 + n, dtype=np.int64)
@@ -156,7 +176,7 @@ class RaggedBatch:
             dv.append(dev_ints[o:o + n])
             o += n
         return RaggedBatch(T, S, mb, dv[0], dv[1], dv[2], dv[3], dv[4], dv[5], dv[6].view(S, mb), torch.from_numpy(slots).to(device),
-                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10], max(1, min(L, max(lens, default=1))))
+                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10], max(1, min(L, max(lens, default=1))), host_blocks)
 
 
 # ------------------------------------------------------------------------------------------------------------------ layer descriptions
@@ -813,7 +833,7 @@ class GatedSinkAttention(_Module):
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
         _call("mrs_hyb_paged_attn_opts", q, src.k_cache, src.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, b.max_blocks,
               0, 0, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, s.softcap, int(s.sink), u[:, self.gate_col:], u.stride(0),
-              *m.key_splits(b, s.heads, s.vdim))
+              *m.key_splits(b, s.heads, s.vdim), 0)
         m.linear(o, self.w_o, out=x, accumulate=accumulate)
 
 
@@ -894,6 +914,7 @@ class LatentAttention(_Module):
         self.w_in = torch.cat([q, dkv], 0).to(dev, dt).contiguous()                                       # [q | latent, W]
         self.w_ukT = uk.reshape(s.heads, s.dim, s.kv_rank).transpose(1, 2).to(dev, dt).contiguous()       # [H, kv_rank, dim]: q' = this . q
         self.w_uv = uv.reshape(s.heads, s.vdim, s.kv_rank).to(dev, dt).contiguous()                       # [H, vdim, kv_rank]
+        self.w_uk = uk.to(dev, dt).contiguous()                                                           # [H * dim, kv_rank]: the keys themselves (prompt steps)
         self.c_norm = self.w(get, p + "dkv.norm", False)
         self.w_o = self.w(get, p + "o", True)
         if self.c_norm.numel() != s.kv_rank or tuple(self.w_o.shape) != (W, s.heads * s.vdim):
@@ -906,12 +927,38 @@ class LatentAttention(_Module):
         u = m.linear(h, self.w_in)                                         # f32 [T, q | latent]
         q = torch.empty(T, H * D, dtype=dt, device=dev)
         _call("mrs_hyb_latent_norm_cache", u, u.stride(0), H * D, R, self.c_norm, b.slot_mapping, q, self.c_cache, m.spec.eps, T, m.dt)
-        qa = m.batched_linear(q, self.w_ukT, H)                            # [T, H * kv_rank] in the serving dtype
-        oa = torch.empty(T, H * R, dtype=dt, device=dev)
-        _call("mrs_hyb_paged_attn_opts", qa, self.c_cache, self.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, m.block_size, b.max_blocks, 0, 0, s.scale,
-              m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, 0, None, 0, *m.key_splits(b, H, R))
-        ov = m.batched_linear(oa, self.w_uv, H)                            # [T, H * vdim]
+        if self.expands(b):
+            # a step with prompt portions: the contexts' latent rows are gathered block by block and expanded into keys and values of `dim` / `vdim` per head (two products
+            # on the matrix cores); attention then costs dim + vdim per (query, key) pair instead of 2 kv_rank
+            tables, source, n = b.context_blocks()
+            bs = m.block_size
+            per = bs * R * self.c_cache.element_size() // 4
+            c = torch.empty(n * bs, R, dtype=dt, device=dev)
+            _call("mrs_hyb_gather_rows", self.c_cache, source, c, n, per)
+            k = m.linear_rounded(c, self.w_uk)                              # [n * bs, H * dim]: block, slot, head -- the attention kernel's token-major layout
+            v = m.linear_rounded(c, self.w_uv.view(H * Dv, R))
+            ov = torch.empty(T, H * Dv, dtype=dt, device=dev)
+            _call("mrs_hyb_paged_attn_opts", q, k, v, tables, b.tok_seq, b.tok_pos, ov, T, H, H, D, Dv, bs, b.max_blocks, 0, 0, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len,
+                  b.segments, RaggedBatch.SEGMENT, 0.0, 0, None, 0, None, 0, 1)
+        else:
+            qa = m.batched_linear(q, self.w_ukT, H)                        # [T, H * kv_rank] in the serving dtype
+            oa = torch.empty(T, H * R, dtype=dt, device=dev)
+            _call("mrs_hyb_paged_attn_opts", qa, self.c_cache, self.c_cache, b.block_tables, b.tok_seq, b.tok_pos, oa, T, H, 1, R, R, m.block_size, b.max_blocks, 0, 0, s.scale,
+                  m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, 0, None, 0, *m.key_splits(b, H, R), 0)
+            ov = m.batched_linear(oa, self.w_uv, H)                        # [T, H * vdim]
         m.linear(ov, self.w_o, out=x, accumulate=accumulate)
+
+    MATRIX_TO_VECTOR_RATE = 6.0   # products on the matrix cores against attention arithmetic on the vector ALU, per operation
+
+    def expands(self, b: RaggedBatch) -> bool:
+        """Whether this step materialises keys and values.  Reading latent rows directly costs 2 kv_rank multiply-adds per (query, key) pair and head, expanded ones dim + vdim
+        plus the expansion of every context row (kv_rank (dim + vdim) per head, on the matrix cores).  With about rows / 2 queries per context row the expansion pays from
+        rows > 2 kv_rank (dim + vdim) / (rate (2 kv_rank - dim - vdim)) on; steps of single rows never expand."""
+        s = self.s
+        gain = 2 * s.kv_rank - s.dim - s.vdim
+        if b.seg_rows <= 1 or b.host_blocks is None or gain <= 0 or (self.m.block_size * s.kv_rank * self.c_cache.element_size()) % 4:
+            return False
+        return b.rows * self.MATRIX_TO_VECTOR_RATE * gain > 2 * s.kv_rank * (s.dim + s.vdim)
 
 
 class GluFeedForward(_Module):
@@ -1062,6 +1109,13 @@ class HybridDecoder:
         if splits < 2:
             return None, 0
         return torch.empty(splits, b.rows, heads, vdim + 2, dtype=torch.float32, device=self.device), splits
+
+    def linear_rounded(self, a, w):
+        """a [M, K] . w [N, K]^T -> [M, N] in the serving dtype, rounded once: a product whose consumer is another product or the attention kernel."""
+        M, K = a.shape
+        out = torch.empty(M, w.shape[0], dtype=self.torch_dtype, device=self.device)
+        _call("mrs_hyb_gemm_batched", a, w, out, M, w.shape[0], K, a.stride(0), w.stride(0), out.stride(0), self.dt, 0, 0, 0, 0, 1)
+        return out
 
     def batched_linear(self, a, w, heads: int):
         """a [M, heads * K] (column block h = the operand of head h), w [heads, N, K] -> [M, heads * N] in the serving dtype, rounded once: per-head products whose

@@ -489,7 +489,7 @@ def test_planted_keys_sink_and_cap(dev, dtype):
             splits = 1 + (i + j0) % 6                         # the keys dealt to several workgroups (some of them without a share), or all to one
         scratch = torch.full((max(splits, 1), n, H, Dv + 2), float("nan"), device=dev) if splits > 1 else None
         _call("mrs_hyb_paged_attn_opts", qq, att.k_cache, att.v_cache, b.block_tables, b.tok_seq, b.tok_pos, out, n, H, G, D, Dv, bs, b.max_blocks, 0, 0, 1.0, m.dt,
-              b.seg_entry, b.seg_row0, b.seg_len, b.segments, 64, cap, sink, gate, H * Dv if gate is not None else 0, scratch, splits if splits > 1 else 0)
+              b.seg_entry, b.seg_row0, b.seg_len, b.segments, 64, cap, sink, gate, H * Dv if gate is not None else 0, scratch, splits if splits > 1 else 0, 0)
         return out[n - 1].double().cpu().view(H, Dv)
     j0 = 0
     for i in (60, 64, 95, 96, 299):
