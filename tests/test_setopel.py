@@ -173,7 +173,7 @@ def _batch(dev, parts, bs=32, blocks=None):
 # ---------------------------------------------------------------------------------------------------------------- no device needed
 def test_config_reader_takes_every_size_and_constant_from_the_file():
     from mistralrs_amd.hybrid import GluSpec, LatentAttentionSpec, RetentionSpec, SinkAttentionSpec, setopel_spec
-    cfg = config([attn(heads=6, kv_heads=3, dim=10, vdim=14, conv=5, cap=11.0, coef=0.5, every=9, mlp=glu(77), scale=0.3),
+    cfg = config([attn(heads=6, kv_heads=3, dim=10, vdim=14, conv=5, cap=11.0, coef=0.75, every=9, mlp=glu(77), scale=0.3),
                   attn(heads=6, kv_heads=3, dim=10, vdim=14, conv=0, cap=0.0, coef=0.0, kv_from=0, mlp=None),
                   ret(heads=3, dim=12, vdim=20, decay=(0.5, 0.75, 0.875), dims=4, base=77.0, mlp="glu"), ret(dims=0),
                   lat(heads=5, dim=6, vdim=7, rank=9, mlp=glu(3), scale=0.7)], vocab=123, width=56, eps=3e-4, streams=4, mult=0.125)
@@ -183,7 +183,7 @@ def test_config_reader_takes_every_size_and_constant_from_the_file():
     assert [l.kind for l in sp.layers] == ["sink_attention", "sink_attention", "retention", "retention", "latent_attention"]
     assert isinstance(a.mixer, SinkAttentionSpec) and isinstance(c.mixer, RetentionSpec) and isinstance(e.mixer, LatentAttentionSpec)
     assert (a.mixer.heads, a.mixer.kv_heads, a.mixer.dim, a.mixer.vdim, a.mixer.scale, a.mixer.conv, a.mixer.softcap, a.mixer.temp_coef, a.mixer.temp_every, a.mixer.kv_from,
-            a.mixer.sink) == (6, 3, 10, 14, 0.3, 5, 11.0, 0.5, 9, None, True)
+            a.mixer.sink) == (6, 3, 10, 14, 0.3, 5, 11.0, 0.75, 9, None, True)
     assert isinstance(a.ff, GluSpec) and a.ff.ff == 77 and b.ff is None
     assert (b.mixer.conv, b.mixer.softcap, b.mixer.temp_every, b.mixer.kv_from) == (0, 0.0, 0, 0)
     assert (c.mixer.heads, c.mixer.dim, c.mixer.vdim, c.mixer.decay, c.mixer.rotary.dims, c.mixer.rotary.base, c.mixer.rotary.layout) == (3, 12, 20, [0.5, 0.75, 0.875], 4, 77.0, "half")
@@ -419,7 +419,7 @@ def test_sink_attention_alone(dev, shape, dtype, bar):
     _alone(attn(mlp=None, **shape), dev, dtype, bar)
 
 
-RET_SHAPES = [dict(), dict(heads=3, dim=10, vdim=7, decay=(0.25, 0.9, 1.0), dims=10), dict(heads=1, dim=32, vdim=24, decay=(0.99609375,), dims=8, base=1e6),
+RET_SHAPES = [dict(), dict(heads=3, dim=10, vdim=7, decay=(0.25, 0.9, 1.0), dims=10), dict(heads=1, dim=32, vdim=24, decay=(0.99609375,), dims=8, base=2e5),
               dict(heads=4, dim=4, vdim=130, decay=(0.5, 0.75, 0.875, 0.9375), dims=0), dict(heads=2, dim=72, vdim=8, dims=2), dict(heads=2, dim=136, vdim=16, dims=136)]
 
 
@@ -634,7 +634,7 @@ def test_first_tokens_see_zeros_not_the_slots_former_owner(dev):
 # ---------------------------------------------------------------------------------------------------------------- whole models (GPU)
 @pytest.mark.gpu
 @pytest.mark.parametrize("dtype,bar", [("float32", 3e-5), ("bfloat16", 4e-2)])
-@pytest.mark.parametrize("streams,mult", [(3, 0.4), (1, 0.7), (0, 0.3), (0, None)], ids=["streams3", "streams1", "scaled", "plain"])
+@pytest.mark.parametrize("streams,mult", [(3, 0.4), (1, 0.7), (0, 0.6), (0, None)], ids=["streams3", "streams1", "scaled", "plain"])
 def test_whole_prompt_every_layer(dev, dtype, bar, streams, mult):
     cfg = config(STACK, streams=streams, mult=mult)
     w = weights(cfg, 5)
@@ -696,7 +696,7 @@ def test_mixed_batches_with_reused_pages_and_slots(dev, dtype, bar):
 
 @pytest.mark.gpu
 def test_long_decoding_past_temperature_steps_and_slow_decays(dev):
-    cfg = config([attn(every=11, conv=4), ret(decay=(0.99951171875, 0.9), dims=8, base=1e4, mlp="glu"), lat(), attn(kv_from=0, every=64, conv=2)])
+    cfg = config([attn(every=11, conv=4), ret(decay=(0.9990234375, 0.9), dims=8, base=1e4, mlp="glu"), lat(), attn(kv_from=0, every=64, conv=2)])
     w = weights(cfg, 8)
     t = toks(260, cfg["vocab"], 16)
     want = O.forward(cfg, f64(w), t)
