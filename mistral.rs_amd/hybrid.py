@@ -820,13 +820,13 @@ class GatedSinkAttention(_Module):
         s, m = self.s, self.m
         T = b.rows
         u = m.linear(h, self.w_in)                                         # f32 [T, q | k | v | gate logits]
-        qb = self.bias[:self.nq]
-        kb, vb = (self.bias[self.nq:self.nq + self.nk], self.bias[self.nq + self.nk:]) if self.own else (None, None)
         q = torch.empty(T, self.nq, dtype=m.torch_dtype, device=m.device)
         if s.conv:   # bias, convolution, temperature and the page write in one launch (the slots' taps in a second one when a portion is in the batch)
             _call("mrs_hyb_conv_qkv_cache", u, u.stride(0), self.bias, self.conv_w, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, b.tok_pos, b.slot_mapping, q,
                   self.k_cache, self.v_cache, T, b.entries, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size, s.conv, s.temp_coef, s.temp_every, m.dt)
         else:
+            qb = self.bias[:self.nq]
+            kb, vb = (self.bias[self.nq:self.nq + self.nk], self.bias[self.nq + self.nk:]) if self.own else (None, None)
             _call("mrs_hyb_qkv_bias_temp_cache", u, u.stride(0), qb, kb, vb, b.tok_pos, b.slot_mapping, q, self.k_cache, self.v_cache, T, s.heads, s.kv_heads, s.dim, s.vdim,
                   m.block_size, s.temp_coef, s.temp_every, m.dt)
         src = self if self.own else m.layers[s.kv_from].mixer               # that layer ran earlier in this step: its pages hold this step's rows already
