@@ -70,10 +70,10 @@ def libraries():
         for s in srcs:
             if os.path.exists(os.path.join(CSRC, s)):
                 libs.setdefault(lib, []).append(_tu(s, os.path.basename(os.path.splitext(s)[0]) + ".o", decode_defs.get(s, ())))
-    # layer-list ("hybrid") decoders in their checkpoint dtype: a library of its own, so that serving such a model compiles five files, not the quantized stack.
+    # layer-list ("hybrid") decoders in their checkpoint dtype: a library of its own, so that serving such a model compiles six files, not the quantized stack.
     # It carries the host-side cache bookkeeping too (the same objects libmrs_hip_ext.so links).
     libs[HYBRID_LIB] = [_tu(s, os.path.basename(os.path.splitext(s)[0]) + ".o", PACKED_FP32_OFF if s.endswith(".hip") else ())
-                        for s in ("hyb_gemm.hip", "hyb_kernels.hip", "hyb_attn_talk.hip", "host/kv_cache_manager.cpp", "host/state_pool.cpp")]
+                        for s in ("hyb_gemm.hip", "hyb_kernels.hip", "hyb_attn_talk.hip", "hyb_recur.hip", "host/kv_cache_manager.cpp", "host/state_pool.cpp")]
     return libs
 
 

@@ -269,8 +269,9 @@ __global__ void __launch_bounds__(256) gemm_tile_f32_kernel(GemmArgs a) {
 //              routed inputs)
 //   IN_GLU_CLAMP  A = f32 [M, 2 K] = gate | up: g = min(gate, p0), u = clamp(up, -p0, p0): x_k = round_T(g sigmoid(p1 g) (u + 1))
 //   IN_BIAS_XIELU A = f32 [M, K]: z = A + in_bias: x_k = round_T(z > 0 ? p0 z^2 + z / 2 : p1 (e^z - 1 - z) + z / 2)
+//   IN_RELU_SQ A = f32 [M, K]: x_k = round_T(max(A, 0)^2)
 // The batched form offsets A by columns: only IN_PLAIN reads it there.
-enum { IN_PLAIN = 0, IN_GLU = 1, IN_SCALED = 2, IN_GLU_CLAMP = 3, IN_BIAS_XIELU = 4 };
+enum { IN_PLAIN = 0, IN_GLU = 1, IN_SCALED = 2, IN_GLU_CLAMP = 3, IN_BIAS_XIELU = 4, IN_RELU_SQ = 5 };
 struct GemvArgs {
   const void *A;
   const void *W;
@@ -326,6 +327,7 @@ template <class T, int IN> __device__ __forceinline__ float act1(const GemvArgs 
   if (IN == IN_GLU) return round_to<T>(silu_in(A[(size_t)m * a.lda + k]) * A[(size_t)m * a.lda + a.K + k]);
   if (IN == IN_GLU_CLAMP) return round_to<T>(glu_clamp_in(A[(size_t)m * a.lda + k], A[(size_t)m * a.lda + a.K + k], a.p0, a.p1));
   if (IN == IN_BIAS_XIELU) return round_to<T>(xielu_in(A[(size_t)m * a.lda + k] + (a.in_bias ? a.in_bias[k] : 0.f), a.p0, a.p1));
+  if (IN == IN_RELU_SQ) { const float v = fmaxf(A[(size_t)m * a.lda + k], 0.f); return round_to<T>(v * v); }
   const int r = a.src_row[m];
   return round_to<T>((a.src_scale ? a.src_scale[r] : 1.0f) * A[(size_t)(r / a.src_div) * a.lda + k]);
 }
@@ -354,6 +356,12 @@ template <class T, int IN> __device__ __forceinline__ void act8(const GemvArgs &
     if (a.in_bias) Vec8<float>::load(a.in_bias + k, bv);
 #pragma unroll
     for (int j = 0; j < 8; ++j) x[j] = round_to<T>(xielu_in(x[j] + (a.in_bias ? bv[j] : 0.f), a.p0, a.p1));
+    return;
+  }
+  if (IN == IN_RELU_SQ) {
+    Vec8<float>::load(A + (size_t)m * a.lda + k, x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) { const float v = fmaxf(x[j], 0.f); x[j] = round_to<T>(v * v); }
     return;
   }
   const int r = a.src_row[m];
@@ -477,11 +485,11 @@ extern "C" int mrs_hyb_gemm_batched(const void *A, const void *W, void *C, int M
 }
 
 /* in_mode: 0 plain (A in dtype), 1 GLU (A = f32 [M, 2 K] gate | up), 2 scaled rows (A = f32 source rows; row m = src_scale[r] * A[r / src_div], r = src_row[m]; no
- * src_scale: the rows are gathered as they are), 3 clamped GLU (A = f32 [M, 2 K]; p0 = limit, p1 = the sigmoid's factor), 4 xIELU(A + in_bias) (p0, p1 = its coefficients) */
+ * src_scale: the rows are gathered as they are), 3 clamped GLU (A = f32 [M, 2 K]; p0 = limit, p1 = the sigmoid's factor), 4 xIELU(A + in_bias) (p0, p1 = its coefficients), 5 max(A, 0)^2 (A = f32 [M, K]) */
 extern "C" int mrs_hyb_gemv_act(const void *A, const void *W, float *C, int M, int N, int K, int lda, int ldw, int ldc, int dtype, int accumulate, const int *row_group,
                                 long long wstride, int in_mode, const int *src_row, const float *src_scale, int src_div, const float *in_bias, float p0, float p1, void *stream) {
   if (M <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2) || in_mode < 0 || in_mode > 4) return fail("mrs_hyb_gemv: bad shape / dtype / input mode");
+  if (K <= 0 || lda < K || ldw < K || ldc < N || (dtype != 1 && dtype != 2) || in_mode < 0 || in_mode > 5) return fail("mrs_hyb_gemv: bad shape / dtype / input mode");
   if ((in_mode == 1 || in_mode == 3) && lda < 2 * K) return fail("mrs_hyb_gemv: the gate | up operand needs rows of 2 K values");
   if (in_mode == 2 && (!src_row || src_div <= 0)) return fail("mrs_hyb_gemv: gathered rows need their source table");
   if (!row_group && M > 8) return fail("mrs_hyb_gemv: at most 8 rows share a weight");
@@ -494,7 +502,7 @@ extern "C" int mrs_hyb_gemv_act(const void *A, const void *W, float *C, int M, i
   hipStream_t s = (hipStream_t)stream;
 #define MRS_GEMV_(T, MR, IN) hipLaunchKernelGGL((gemv_rows_kernel<T, MR, IN>), grid, dim3(256), 0, s, a)
 #define MRS_GEMV(T, MR) do { if (in_mode == 0) MRS_GEMV_(T, MR, IN_PLAIN); else if (in_mode == 1) MRS_GEMV_(T, MR, IN_GLU); else if (in_mode == 2) MRS_GEMV_(T, MR, IN_SCALED); \
-                             else if (in_mode == 3) MRS_GEMV_(T, MR, IN_GLU_CLAMP); else MRS_GEMV_(T, MR, IN_BIAS_XIELU); } while (0)
+                             else if (in_mode == 3) MRS_GEMV_(T, MR, IN_GLU_CLAMP); else if (in_mode == 4) MRS_GEMV_(T, MR, IN_BIAS_XIELU); else MRS_GEMV_(T, MR, IN_RELU_SQ); } while (0)
   const int mr = row_group ? 1 : M;
   if (dtype == 1) { if (mr <= 1) MRS_GEMV(mrs::bf16_t, 1); else if (mr <= 2) MRS_GEMV(mrs::bf16_t, 2); else if (mr <= 4) MRS_GEMV(mrs::bf16_t, 4); else MRS_GEMV(mrs::bf16_t, 8); }
   else { if (mr <= 1) MRS_GEMV(float, 1); else if (mr <= 2) MRS_GEMV(float, 2); else if (mr <= 4) MRS_GEMV(float, 4); else MRS_GEMV(float, 8); }

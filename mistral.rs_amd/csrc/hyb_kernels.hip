@@ -227,6 +227,8 @@ struct ScanArgs {
   float *carry;       // [segments, heads, N, P]: L_k, then init_(k+1)
   float *decay;       // [segments, heads]: d_k
   int C, ldu, dt_col, heads, P, N, G, rows;
+  int Pin;            // value columns that xbc carries per head; P - Pin (0 or 1) further columns of the state take x = 1 (a running sum of dt B next to the outer products)
+  int ext_steps;      // `steps` was filled by the caller (gates of another form): nothing of dt_bias / A_log / fixed_decay is read
 };
 __global__ void __launch_bounds__(256) ssd_steps_kernel(ScanArgs a) {
   const int i = blockIdx.x * 256 + threadIdx.x;
@@ -267,7 +269,8 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
   if (len <= 0 || (LOCAL && last)) return;
   const bool live = p < a.P;
   const int pc = live ? p : a.P - 1;
-  const int g = h / (a.heads / a.G), inner = a.heads * a.P;
+  const int g = h / (a.heads / a.G), inner = a.heads * a.Pin, inner_out = a.heads * a.P;
+  const bool one_col = pc >= a.Pin;
   int nk = a.N - r * K;  // this lane's rows n = r K + k, k < nk
   nk = nk < 0 ? 0 : (nk > K ? K : nk);
   const size_t np = (size_t)a.N * a.P;
@@ -303,9 +306,9 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
         C_[k] = k < nk ? cv : 0.f;
       }
     }
-    g_.x = xr[h * a.P + pc];
+    g_.x = one_col ? 1.0f : xr[h * a.Pin + pc];
     float d0, d1;
-    if (DEPTH == 1 && !LOCAL) {  // decode steps: the step size and decay inline (ssd_steps_kernel's expressions), one launch less
+    if (DEPTH == 1 && !LOCAL && !a.ext_steps) {  // decode steps: the step size and decay inline (ssd_steps_kernel's expressions), one launch less
       if (a.fixed_decay) { d0 = 1.0f; d1 = a.fixed_decay[h]; }
       else {
         d0 = softplus_f(a.u[(size_t)row * a.ldu + a.dt_col + h] + a.dt_bias[h]);
@@ -336,7 +339,7 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
       if (!LOCAL) {
 #pragma unroll
         for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
-        if (r == 0 && live && i < len) a.out[(size_t)(r0 + i) * inner + h * a.P + p] = fmaf(Dh, xv, part);
+        if (r == 0 && live && i < len) a.out[(size_t)(r0 + i) * inner_out + h * a.P + p] = fmaf(Dh, xv, part);
       }
     }
   }
@@ -364,7 +367,7 @@ template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_b
   if (len <= 0 || (LOCAL && last)) return;
   const bool live = p < a.P;
   const int pc = live ? p : a.P - 1;
-  const int g = h / (a.heads / a.G), inner = a.heads * a.P, N = a.N, P = a.P;
+  const int g = h / (a.heads / a.G), inner = a.heads * a.Pin, inner_out = a.heads * a.P, N = a.N, P = a.P;
   int nk = N - r * K;
   nk = nk < 0 ? 0 : (nk > K ? K : nk);
   const size_t np = (size_t)N * P;
@@ -386,7 +389,7 @@ template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_b
         const float *xr = a.xbc + (size_t)row * a.C;
         if (j < N) v = xr[bcol + j];
         else if (j < 2 * N) v = xr[ccol + j - N];
-        else if (j < 2 * N + P) v = xr[h * P + j - 2 * N];
+        else if (j < 2 * N + P) v = j - 2 * N < a.Pin ? xr[h * a.Pin + j - 2 * N] : 1.0f;
         else v = a.steps[2 * ((size_t)row * a.heads + h) + (j - 2 * N - P)];
       }
       stg[q] = v;
@@ -439,7 +442,7 @@ template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_b
       else {
 #pragma unroll
         for (int m = 1; m < R; m <<= 1) part += __shfl_xor(part, m, 64);
-        if (r == 0 && live) a.out[(size_t)(r0 + c0 + j) * inner + h * P + p] = fmaf(Dh, xv, part);
+        if (r == 0 && live) a.out[(size_t)(r0 + c0 + j) * inner_out + h * P + p] = fmaf(Dh, xv, part);
       }
     }
     if (more) put(sm + (flip ^ 1) * per);
@@ -466,19 +469,30 @@ struct QkArgs {
   void *k_cache, *v_cache;  // [blocks, G, block_size, D | Dv] in T
   int ld, H, G, D, Dv, rot, block_size;
   float eps;
+  int per_head;       // the norm runs over every head's D values with weights [D] shared by the heads, instead of over the whole projection with weights [H * D]
 };
 template <class T> __global__ void __launch_bounds__(256) qk_norm_rope_cache_kernel(QkArgs a) {
   __shared__ float red[4];
+  extern __shared__ float head_inv[];  // per_head: 1 / rms of every query and key head
   const int t = blockIdx.x, tid = threadIdx.x;
   const int nq = a.H * a.D, nk = a.G * a.D, nv = a.G * a.Dv;
   const float *q = a.qkv + (size_t)t * a.ld, *k = q + nq, *v = k + nk;
   float iq = 1.f, ik = 1.f;
-  if (a.qw) {
+  if (a.per_head) {
+    for (int j = tid >> 6; j < a.H + a.G; j += 4) {
+      const float *src = q + (size_t)j * a.D;  // key heads follow the query heads in the row
+      float s = 0.f;
+      for (int d = tid & 63; d < a.D; d += 64) s = fmaf(src[d], src[d], s);
+      s = wave_sum(s);
+      if ((tid & 63) == 0) head_inv[j] = ((j < a.H ? a.qw : a.kw) != nullptr) ? 1.0f / sqrtf(s / (float)a.D + a.eps) : 1.0f;
+    }
+    __syncthreads();
+  } else if (a.qw) {
     float s = 0.f;
     for (int c = tid; c < nq; c += 256) s = fmaf(q[c], q[c], s);
     iq = 1.0f / sqrtf(block_sum_256(s, red) / (float)nq + a.eps);
   }
-  if (a.kw) {
+  if (a.kw && !a.per_head) {
     float s = 0.f;
     for (int c = tid; c < nk; c += 256) s = fmaf(k[c], k[c], s);
     ik = 1.0f / sqrtf(block_sum_256(s, red) / (float)nk + a.eps);
@@ -492,11 +506,11 @@ template <class T> __global__ void __launch_bounds__(256) qk_norm_rope_cache_ker
     const bool is_q = e2 < nq / 2;
     const int e = is_q ? 2 * e2 : 2 * e2 - nq;
     const float *src = is_q ? q : k;
-    const float inv = is_q ? iq : ik;
     const float *w = is_q ? a.qw : a.kw;
-    float x0 = src[e] * inv, x1 = src[e + 1] * inv;
-    if (w) { x0 *= w[e]; x1 *= w[e + 1]; }
     const int d = e % a.D;
+    const float inv = a.per_head ? head_inv[(is_q ? 0 : a.H) + e / a.D] : (is_q ? iq : ik);
+    float x0 = src[e] * inv, x1 = src[e + 1] * inv;
+    if (w) { x0 *= w[a.per_head ? d : e]; x1 *= w[a.per_head ? d + 1 : e + 1]; }
     if (d < a.rot) {
       float sn, cs;
       sincosf(pos * a.freq[d >> 1], &sn, &cs);
@@ -538,7 +552,14 @@ struct AttnArgs {
   float *scratch;
   int splits, rows;
   int token_major;      // K / V rows laid out [block, slot, kv head, dim] (a product's row-major output) instead of [block, kv head, slot, dim]
+  int chunk;            // > 0: position i sees j <= i only inside its own chunk, floor(i / chunk) == floor(j / chunk), chunks counted from position 0 (window / keep_first unused)
+  const float *sink_logit;  // [H], nullable: with `sink`, the extra term of head h is e^{sink_logit[h]} instead of e^0
+  int gate_per_head;    // the gate holds ONE logit per (row, head) at column h (ldg >= H) instead of one per output value
 };
+__device__ __forceinline__ float sink_of(const AttnArgs &a, int h) { return a.sink_logit ? a.sink_logit[h] : 0.f; }
+__device__ __forceinline__ const float *gate_row(const AttnArgs &a, int t, int h) {
+  return a.gate ? a.gate + (size_t)t * a.ldg + (a.gate_per_head ? (size_t)h : (size_t)h * a.Dv) : nullptr;
+}
 __device__ __forceinline__ long long kv_row(const AttnArgs &a, const int *bt, int key, int g) {
   const long long blk = bt[key / a.block_size];
   const int off = key % a.block_size;
@@ -578,8 +599,9 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
   const int *bt = a.block_tables + (size_t)s * a.max_blocks;
   int w_lo = a.window > 0 ? i - a.window + 1 : 0;
   if (w_lo < 0) w_lo = 0;
+  if (a.chunk > 0) w_lo = (i / a.chunk) * a.chunk;
   int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;  // kept first tokens that the window does not already cover
-  if (n1 < 0) n1 = 0;
+  if (n1 < 0 || a.chunk > 0) n1 = 0;
   int total = n1 + (i - w_lo + 1), v_begin = 0;
   const bool split = a.splits > 1;
   if (split) {  // this workgroup's share of the passes
@@ -588,7 +610,7 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
     const int v_end = v_begin + per * 64;
     total = total < v_end ? total : v_end;
   }
-  float m = (a.sink && !split) ? 0.f : -FLT_MAX, l = (a.sink && !split) ? 1.f : 0.f, o[DVC][2];
+  float m = (a.sink && !split) ? sink_of(a, h) : -FLT_MAX, l = (a.sink && !split) ? 1.f : 0.f, o[DVC][2];
 #pragma unroll
   for (int c = 0; c < DVC; ++c) o[c][0] = o[c][1] = 0.f;
   MRS_WAVE_SYNC();
@@ -663,12 +685,13 @@ template <class T, int DVC, bool VEC> __global__ void __launch_bounds__(64) page
   }
   const float inv = 1.0f / l;
   T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
-  const float *gr = a.gate ? a.gate + (size_t)t * a.ldg + (size_t)h * a.Dv : nullptr;
+  const float *gr = gate_row(a, t, h);
+  const int gs = a.gate_per_head ? 0 : 1;
 #pragma unroll
   for (int c = 0; c < DVC; ++c) {
     const int d = 128 * c + 2 * lane;
-    if (d < a.Dv) out[d] = from_f<T>(o[c][0] * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
-    if (d + 1 < a.Dv) out[d + 1] = from_f<T>(o[c][1] * inv * (gr ? sigmoid_f(gr[d + 1]) : 1.0f));
+    if (d < a.Dv) out[d] = from_f<T>(o[c][0] * inv * (gr ? sigmoid_f(gr[gs * d]) : 1.0f));
+    if (d + 1 < a.Dv) out[d + 1] = from_f<T>(o[c][1] * inv * (gr ? sigmoid_f(gr[gs * (d + 1)]) : 1.0f));
   }
 }
 // joins the splits of a row and head: M = max_s m_s (and 0 with the sink), L = sum_s l_s e^{m_s - M} (+ e^{-M}), out = sum_s o_s e^{m_s - M} / L (times sigmoid(gate))
@@ -676,17 +699,18 @@ template <class T> __global__ void __launch_bounds__(64) attn_merge_kernel(AttnA
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, stride = a.Dv + 2;
   const float *base = a.scratch + ((size_t)t * a.H + h) * stride;
   const size_t step = (size_t)a.rows * a.H * stride;
-  float M = a.sink ? 0.f : -FLT_MAX;
+  const float sv = sink_of(a, h);
+  float M = a.sink ? sv : -FLT_MAX;
   for (int s = 0; s < a.splits; ++s) M = fmaxf(M, base[s * step + a.Dv]);
-  float L = a.sink ? expf(-M) : 0.f;
+  float L = a.sink ? expf(sv - M) : 0.f;
   for (int s = 0; s < a.splits; ++s) L += base[s * step + a.Dv + 1] * expf(base[s * step + a.Dv] - M);
   const float inv = 1.0f / L;
   T *out = (T *)a.out + ((size_t)t * a.H + h) * a.Dv;
-  const float *gr = a.gate ? a.gate + (size_t)t * a.ldg + (size_t)h * a.Dv : nullptr;
+  const float *gr = gate_row(a, t, h);
   for (int d = lane; d < a.Dv; d += 64) {
     float acc = 0.f;
     for (int s = 0; s < a.splits; ++s) acc = fmaf(base[s * step + d], expf(base[s * step + a.Dv] - M), acc);
-    out[d] = from_f<T>(acc * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
+    out[d] = from_f<T>(acc * inv * (gr ? sigmoid_f(gr[a.gate_per_head ? 0 : d]) : 1.0f));
   }
 }
 
@@ -712,13 +736,14 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
   const int *bt = a.block_tables + (size_t)s * a.max_blocks;
   int w_lo = a.window > 0 ? i0 - a.window + 1 : 0;
   if (w_lo < 0) w_lo = 0;
+  if (a.chunk > 0) w_lo = (i0 / a.chunk) * a.chunk;   // the first query's chunk; a later query of the tile may start a new one and then sees only part of the range
   int n1 = a.keep_first < w_lo ? a.keep_first : w_lo;
-  if (n1 < 0) n1 = 0;
+  if (n1 < 0 || a.chunk > 0) n1 = 0;
   const int total = n1 + (i0 + nq - 1 - w_lo + 1);
   float m[NQ], l[NQ], o[NQ][DVC][2];
 #pragma unroll
   for (int q = 0; q < NQ; ++q) {
-    m[q] = a.sink ? 0.f : -FLT_MAX; l[q] = a.sink ? 1.f : 0.f;
+    m[q] = a.sink ? sink_of(a, h) : -FLT_MAX; l[q] = a.sink ? 1.f : 0.f;
 #pragma unroll
     for (int c = 0; c < DVC; ++c) o[q][c][0] = o[q][c][1] = 0.f;
   }
@@ -751,7 +776,7 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
 #pragma unroll
     for (int q = 0; q < NQ; ++q) {
       const int iq = i0 + q;
-      const bool vis = key >= 0 && q < nq && key <= iq && (a.window <= 0 || iq - key < a.window || key < a.keep_first);
+      const bool vis = key >= 0 && q < nq && key <= iq && (a.chunk > 0 ? key >= (iq / a.chunk) * a.chunk : (a.window <= 0 || iq - key < a.window || key < a.keep_first));
       const float sv = vis ? capped(sc[q] * a.scale, a.softcap) : -FLT_MAX;
       const float mn = fmaxf(m[q], wave_max(sv));
       const float alpha = expf(m[q] - mn);
@@ -794,13 +819,14 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
     if (q >= nq) break;
     const float inv = 1.0f / l[q];
     T *out = (T *)a.out + ((size_t)(t0 + q) * a.H + h) * a.Dv;
-    const float *gr = a.gate ? a.gate + (size_t)(t0 + q) * a.ldg + (size_t)h * a.Dv : nullptr;
+    const float *gr = gate_row(a, t0 + q, h);
+    const int gs = a.gate_per_head ? 0 : 1;
 #pragma unroll
     for (int c = 0; c < DVC; ++c) {
       const int d = 128 * c + 2 * lane;
       if (d < a.Dv) {
-        out[d] = from_f<T>(o[q][c][0] * inv * (gr ? sigmoid_f(gr[d]) : 1.0f));
-        out[d + 1] = from_f<T>(o[q][c][1] * inv * (gr ? sigmoid_f(gr[d + 1]) : 1.0f));
+        out[d] = from_f<T>(o[q][c][0] * inv * (gr ? sigmoid_f(gr[gs * d]) : 1.0f));
+        out[d + 1] = from_f<T>(o[q][c][1] * inv * (gr ? sigmoid_f(gr[gs * (d + 1)]) : 1.0f));
       }
     }
   }
@@ -809,9 +835,11 @@ template <class T, int DVC, int NQ> __global__ void __launch_bounds__(64) paged_
 // ---------------------------------------------------------------------------------- mixture of experts: routing, dispatch, gather, GLU, combine
 // Router: one workgroup per row.  logits z_e = w_e . h in f32 (a wave per expert, lanes over the width, butterfly sum); the `top` largest (ties: the lower index).
 // SOFTMAX false: score = sigmoid(z), weights = the scores, un-renormalised; row E of the weight (when has_gate) is the shared expert's gate: gate[t] = sigmoid(w_E . h).
-// SOFTMAX true: score = softmax(z) over ALL experts, weights = out_scale * the chosen scores, un-renormalised.
+// SOFTMAX true: score = softmax(z) over ALL experts, weights = out_scale * the chosen scores, un-renormalised; with `chosen_only` the softmax runs over the chosen logits
+// alone (the weights of a row sum to out_scale).  bias (nullable, [E]) is added to the logits.
 template <bool SOFTMAX> __global__ void __launch_bounds__(1024) route_topk_kernel(const float *__restrict__ h, const float *__restrict__ wr, int W, int E, int top, int has_gate,
-                                                                                  int *__restrict__ ids, float *__restrict__ wts, float *__restrict__ gate, float out_scale) {
+                                                                                  int *__restrict__ ids, float *__restrict__ wts, float *__restrict__ gate, float out_scale,
+                                                                                  const float *__restrict__ bias, int chosen_only) {
   extern __shared__ float z[];  // [E + 1]
   const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float *hr = h + (size_t)t * W;
@@ -829,13 +857,13 @@ template <bool SOFTMAX> __global__ void __launch_bounds__(1024) route_topk_kerne
       for (int k = lane; k < W; k += 64) acc = fmaf(hr[k], w[k], acc);
     }
     acc = wave_sum(acc);
-    if (lane == 0) z[e] = acc;
+    if (lane == 0) z[e] = (bias && e < E) ? acc + bias[e] : acc;
   }
   __syncthreads();
   if (wave != 0) return;
   if (has_gate && lane == 0) gate[t] = sigmoid_f(z[E]);
   float zmax = 0.f, zden = 1.f;
-  if (SOFTMAX) {
+  if (SOFTMAX && !chosen_only) {
     float mx = -FLT_MAX;
     for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
     zmax = wave_max(mx);
@@ -854,11 +882,17 @@ template <bool SOFTMAX> __global__ void __launch_bounds__(1024) route_topk_kerne
       const int oe = __shfl_xor(be, m, 64);
       if (ov > bv || (ov == bv && oe < be)) { bv = ov; be = oe; }
     }
+    if (SOFTMAX && chosen_only && k == 0) zmax = bv;  // the largest logit comes first
     if (lane == 0) {
       ids[(size_t)t * top + k] = be;
-      wts[(size_t)t * top + k] = SOFTMAX ? out_scale * (expf(bv - zmax) / zden) : sigmoid_f(bv);
+      wts[(size_t)t * top + k] = SOFTMAX ? (chosen_only ? expf(bv - zmax) : out_scale * (expf(bv - zmax) / zden)) : sigmoid_f(bv);
     }
     if ((be & 63) == lane) z[be] = -FLT_MAX;  // taken: written by the lane that reads this entry in the next round (every lane holds the same `be` after the butterfly)
+  }
+  if (SOFTMAX && chosen_only && lane == 0) {
+    float den = 0.f;
+    for (int k = 0; k < top; ++k) den += wts[(size_t)t * top + k];
+    for (int k = 0; k < top; ++k) wts[(size_t)t * top + k] = out_scale * (wts[(size_t)t * top + k] / den);
   }
 }
 // stable counting sort of the routes by expert, one workgroup per expert: bounds [E + 1], sorted_route [R] (route index = token * top + k), route_pos [R] (its inverse),
@@ -1217,15 +1251,19 @@ extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const
  * decay [segments, heads] are scratch that is only touched when some entry has more than one segment (segments > entries). */
 static int scan_launch(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, const float *fixed_decay, float *state, float *out,
                        const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry,
-                       float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream) {
+                       float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream, int ones = 0,
+                       int ext_steps = 0) {
   if (entries <= 0 || rows <= 0 || segments <= 0) return 0;
   if (heads <= 0 || G <= 0 || heads % G || P <= 0 || N <= 0) return fail("mrs_hyb_ssd_scan: bad head / group sizes");
   if (segments > 65535 || entries > 65535) return fail("mrs_hyb_ssd_scan: more than 65535 segments in one step");
   if (segments > entries && (!carry || !decay)) return fail("mrs_hyb_ssd_scan: segmented entries need the carry scratch");
-  ScanArgs a{xbc, u, dt_bias, A_log, D, fixed_decay, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows};
-  const bool vec = C % 4 == 0 && (heads * P) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
+  const int Pin = P;  // value columns the rows carry; the state has `ones` more
+  P += ones ? 1 : 0;
+  ScanArgs a{xbc, u, dt_bias, A_log, D, fixed_decay, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows,
+             Pin, ext_steps ? 1 : 0};
+  const bool vec = C % 4 == 0 && (heads * Pin) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
   const bool single = rows == segments;  // one row per segment (decode steps): no ring, step sizes inline
-  if (!single) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
+  if (!single && !ext_steps) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
   const bool split = segments > entries;
 #define MRS_SCAN_(R, K, V, DP, L) hipLaunchKernelGGL((ssd_scan_kernel<R, K, V, DP, L>), dim3((P + 64 / R - 1) / (64 / R), heads, segments), dim3(64), 0, S_(stream), a)
 #define MRS_SCAN_LDS_(R, K, V, L) do { if (nw <= 4) hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 256>), dim3(1, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); \
@@ -1276,16 +1314,40 @@ extern "C" int mrs_hyb_decay_scan(const float *xkq, int ld, const float *fixed_d
                      entries, segments, ld, 0, 0, heads, P, N, G, stream);
 }
 
+/* The same recurrence with step values the caller computed: steps [rows, heads, 2] = (what the state takes in, what it keeps) per row and head, S <- keep S + take k v^T,
+ * o = S^T q; xkq [rows, ld] holds v [heads * P] | k [G * N] | q [G * N] from column 0.  ones != 0: the state has one more column per head that takes v = 1 (the running sum
+ * of take * k beside the outer products): state [slots, heads, N, P + 1], out [rows, heads * (P + 1)], the last value of every head being that column's read-out. */
+extern "C" int mrs_hyb_gated_scan(const float *xkq, int ld, float *steps, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry,
+                                  const int *seg_row0, const int *seg_len, const int *ent_seg0, float *carry, float *decay, int rows, int entries, int segments,
+                                  int heads, int P, int N, int G, int ones, void *stream) {
+  if (!steps) return fail("mrs_hyb_gated_scan: the rows' step values are needed");
+  if (ld < heads * P + 2 * G * N) return fail("mrs_hyb_gated_scan: rows shorter than v | k | q");
+  return scan_launch(xkq, nullptr, nullptr, nullptr, nullptr, nullptr, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, steps, carry, decay, rows,
+                     entries, segments, ld, 0, 0, heads, P, N, G, stream, ones, 1);
+}
+
+static int qk_launch(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping, void *q_out,
+                     void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype, int per_head, void *stream) {
+  if (rows <= 0) return 0;
+  if ((D & 1) || (rot & 1) || rot > D || rot < 0 || H <= 0 || G <= 0 || H % G) return fail("mrs_hyb_qk_norm_rope_cache: head sizes (even dim, even rot <= dim, heads % kv_heads == 0)");
+  QkArgs a{qkv, qw, kw, freq, tok_pos, slot_mapping, q_out, k_cache, v_cache, ld, H, G, D, Dv, rot, block_size, eps, per_head ? 1 : 0};
+  const size_t lds = per_head ? (size_t)(H + G) * 4 : 0;
+  if (lds > 32768) return fail("mrs_hyb_qk_norm_rope_cache: more than 8192 heads");
+  if (dtype == 1) hipLaunchKernelGGL(qk_norm_rope_cache_kernel<mrs::bf16_t>, dim3(rows), dim3(256), lds, S_(stream), a);
+  else if (dtype == 2) hipLaunchKernelGGL(qk_norm_rope_cache_kernel<float>, dim3(rows), dim3(256), lds, S_(stream), a);
+  else return fail("mrs_hyb_qk_norm_rope_cache: dtype");
+  return ok_or("mrs_hyb_qk_norm_rope_cache");
+}
 extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping,
                                           void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype,
                                           void *stream) {
-  if (rows <= 0) return 0;
-  if ((D & 1) || (rot & 1) || rot > D || rot < 0 || H <= 0 || G <= 0 || H % G) return fail("mrs_hyb_qk_norm_rope_cache: head sizes (even dim, even rot <= dim, heads % kv_heads == 0)");
-  QkArgs a{qkv, qw, kw, freq, tok_pos, slot_mapping, q_out, k_cache, v_cache, ld, H, G, D, Dv, rot, block_size, eps};
-  if (dtype == 1) hipLaunchKernelGGL(qk_norm_rope_cache_kernel<mrs::bf16_t>, dim3(rows), dim3(256), 0, S_(stream), a);
-  else if (dtype == 2) hipLaunchKernelGGL(qk_norm_rope_cache_kernel<float>, dim3(rows), dim3(256), 0, S_(stream), a);
-  else return fail("mrs_hyb_qk_norm_rope_cache: dtype");
-  return ok_or("mrs_hyb_qk_norm_rope_cache");
+  return qk_launch(qkv, ld, qw, kw, freq, tok_pos, slot_mapping, q_out, k_cache, v_cache, rows, H, G, D, Dv, rot, block_size, eps, dtype, 0, stream);
+}
+/* the same with the query / key norm per head: every head's D values are divided by their own root mean square and multiplied by qw / kw [D], shared by the heads */
+extern "C" int mrs_hyb_qk_headnorm_rope_cache(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping,
+                                              void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype,
+                                              void *stream) {
+  return qk_launch(qkv, ld, qw, kw, freq, tok_pos, slot_mapping, q_out, k_cache, v_cache, rows, H, G, D, Dv, rot, block_size, eps, dtype, 1, stream);
 }
 
 /* seg_entry / seg_row0 / seg_len [segments] (nullable): the batch's segment table (rows of one entry in pieces); with it, batches that bring portions run the
@@ -1293,11 +1355,13 @@ extern "C" int mrs_hyb_qk_norm_rope_cache(const float *qkv, int ld, const float 
 static int attn_launch(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
                        int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int window, int keep_first, float scale, int dtype,
                        const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *gate, int ldg,
-                       float *scratch, int splits, int token_major, void *stream) {
+                       float *scratch, int splits, int token_major, void *stream, int chunk = 0, const float *sink_logit = nullptr, int gate_per_head = 0) {
   if (rows <= 0) return 0;
   if (Dv > 512 || H % G) return fail("mrs_hyb_paged_window_attn: value size above 512 / heads % kv_heads");
-  if (gate && ldg < H * Dv) return fail("mrs_hyb_paged_window_attn: gate rows shorter than heads * value size");
-  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg, nullptr, 0, rows, token_major ? 1 : 0};
+  if (gate && ldg < (gate_per_head ? H : H * Dv)) return fail("mrs_hyb_paged_window_attn: gate rows shorter than heads (* value size)");
+  if (chunk > 0 && (window > 0 || keep_first > 0)) return fail("mrs_hyb_paged_window_attn: chunks and a sliding window exclude each other");
+  AttnArgs a{q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, H, G, D, Dv, block_size, max_blocks, window, keep_first, scale, softcap > 0.f ? softcap : 0.f, sink ? 1 : 0, gate, ldg, nullptr, 0, rows, token_major ? 1 : 0,
+             chunk > 0 ? chunk : 0, sink ? sink_logit : nullptr, gate_per_head ? 1 : 0};
   const bool vec = D % 8 == 0 && Dv % 2 == 0 && ((uintptr_t)k_cache % 16) == 0 && ((uintptr_t)v_cache % 8) == 0;
   const int c = (Dv + 127) / 128;
   if (vec && seg_entry && segments > 0 && rows > segments && segments <= 65535 && seg_rows > 0) {
@@ -1350,11 +1414,21 @@ extern "C" int mrs_hyb_paged_attn_opts(const void *q, const void *k_cache, const
                      segments, seg_rows, softcap, sink, gate, ldg, scratch, splits, token_major, stream);
 }
 
+/* the same attention inside position chunks (chunk > 0: query i reads the keys j <= i with floor(j / chunk) == floor(i / chunk)), with a learned sink (sink_logit [H], nullable:
+ * the softmax's extra term of head h is e^{sink_logit[h]}) and a gate of one logit per (row, head) (gate_per_head != 0: gate[t * ldg + h]) */
+extern "C" int mrs_hyb_paged_attn_chunked(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out,
+                                          int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int chunk, float scale, int dtype, const int *seg_entry,
+                                          const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *sink_logit, const float *gate,
+                                          int ldg, int gate_per_head, float *scratch, int splits, void *stream) {
+  return attn_launch(q, k_cache, v_cache, block_tables, tok_seq, tok_pos, out, rows, H, G, D, Dv, block_size, max_blocks, 0, 0, scale, dtype, seg_entry, seg_row0, seg_len,
+                     segments, seg_rows, softcap, sink, gate, ldg, scratch, splits, 0, stream, chunk, sink_logit, gate_per_head);
+}
+
 /* h [rows, W] f32 (contiguous), wr [E (+ 1), W] f32 */
 extern "C" int mrs_hyb_route_sigmoid_topk(const float *h, const float *wr, int rows, int W, int E, int top, int has_gate, int *ids, float *wts, float *gate, void *stream) {
   if (rows <= 0) return 0;
   if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_sigmoid_topk: 1 <= top <= experts <= 8192");
-  hipLaunchKernelGGL(route_topk_kernel<false>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate, 1.0f);
+  hipLaunchKernelGGL(route_topk_kernel<false>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, has_gate, ids, wts, gate, 1.0f, (const float *)nullptr, 0);
   return ok_or("mrs_hyb_route_sigmoid_topk");
 }
 
@@ -1362,8 +1436,16 @@ extern "C" int mrs_hyb_route_sigmoid_topk(const float *h, const float *wr, int r
 extern "C" int mrs_hyb_route_softmax_topk(const float *h, const float *wr, int rows, int W, int E, int top, float scale, int *ids, float *wts, void *stream) {
   if (rows <= 0) return 0;
   if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_softmax_topk: 1 <= top <= experts <= 8192");
-  hipLaunchKernelGGL(route_topk_kernel<true>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, 0, ids, wts, (float *)nullptr, scale);
+  hipLaunchKernelGGL(route_topk_kernel<true>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, 0, ids, wts, (float *)nullptr, scale, (const float *)nullptr, 0);
   return ok_or("mrs_hyb_route_softmax_topk");
+}
+
+/* logits = wr h + bias (bias nullable); the `top` largest; weights = scale * softmax over the chosen logits only */
+extern "C" int mrs_hyb_route_topk_softmax(const float *h, const float *wr, const float *bias, int rows, int W, int E, int top, float scale, int *ids, float *wts, void *stream) {
+  if (rows <= 0) return 0;
+  if (top < 1 || top > E || E > 8192) return fail("mrs_hyb_route_topk_softmax: 1 <= top <= experts <= 8192");
+  hipLaunchKernelGGL(route_topk_kernel<true>, dim3(rows), dim3(1024), (size_t)(E + 1) * 4, S_(stream), h, wr, W, E, top, 0, ids, wts, (float *)nullptr, scale, bias, 1);
+  return ok_or("mrs_hyb_route_topk_softmax");
 }
 
 extern "C" int mrs_hyb_moe_dispatch(const int *ids, int R, int E, int *bounds, int *sorted_route, int *route_pos, int *sorted_expert, void *stream) {

@@ -1,0 +1,423 @@
+// hyb_recur.hip -- kernels of the recurrent mixers that write their state with a correction (delta rule) or through exponential gates with a running stabiliser, and
+// of layers whose two sublayers read two norms of the same residual row.  Same conventions as hyb_kernels.hip: a step's rows are one flat range, entry s owns rows
+// [seq_start[s], seq_start[s + 1]) at positions seq_pos0[s] + i and state slot seq_slot[s]; an entry whose first position is 0 reads its slot as zero.
+//
+//   norm pair            one root mean square, two weights: the inputs of a layer's mixer and feed-forward in one pass over the residual row
+//   delta prep           unit-length queries and keys per head, write strengths, decays per head or per (head, key channel)
+//   delta scan           S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q            (f32 state [slot, head, D, Dv])
+//   exponential gates    capped log gates, the running maximum m, the step values e^{i - m'}, e^{f + m - m'} and e^{-m'} of every row
+//   head norm + gate     per-head output norm (optionally behind a normaliser column), shared or full weight, sigmoid / SiLU gate, rounded once for the out-projection
+//   normed average       x (+)= c (y1 / rms(y1) w1 + y2 / rms(y2) w2)
+//   squared ReLU, rounded column blocks
+//
+// Everything here is f32 arithmetic on f32 operands; T is only the type the results are rounded to for the next product.
+#include "common.cuh"
+#include <float.h>
+
+namespace mrs {
+namespace hybr {
+
+static thread_local char g_err[256];
+static int fail(const char *m) { snprintf(g_err, sizeof g_err, "%s", m); return 1; }
+static int ok_or(const char *what) {
+  if (hipGetLastError() == hipSuccess) return 0;
+  snprintf(g_err, sizeof g_err, "%s: launch failed", what);
+  return 1;
+}
+__device__ __forceinline__ float block_sum_256(float v, float *red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
+__device__ __forceinline__ float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
+
+// ---------------------------------------------------------------------------------- x / rms(x) times two weights
+template <class T> __global__ void __launch_bounds__(256) rmsnorm_pair_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ w1, const float *__restrict__ w2,
+                                                                               T *__restrict__ out1, T *__restrict__ out2, float *__restrict__ out2_32, int W, float eps, int one_plus) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float *xr = x + (size_t)t * ldx;
+  float s = 0.f;
+  for (int c = threadIdx.x; c < W; c += 256) s = fmaf(xr[c], xr[c], s);
+  const float inv = 1.0f / sqrtf(block_sum_256(s, red) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = xr[c] * inv, a = v * (one_plus ? 1.0f + w1[c] : w1[c]), b = v * (one_plus ? 1.0f + w2[c] : w2[c]);
+    out1[(size_t)t * W + c] = from_f<T>(a);
+    out2[(size_t)t * W + c] = from_f<T>(b);
+    if (out2_32) out2_32[(size_t)t * W + c] = b;
+  }
+}
+
+// ---------------------------------------------------------------------------------- delta rule: operands of the recurrence
+// c [rows, ldc]: q [G * D] | k [G * D] | v ... after convolution + SiLU; q and k are made unit vectors per head in place (x / sqrt(sum x^2 + 1e-6)), q times D^(-1/2).
+// beta [rows, H] = sigmoid(u[b_col + h]).  Decays [rows, ndec], ndec = H * per: exp(-exp(A_log[c / per]) softplus(a[c] + dt_bias[c])), the rows of `a` being a [rows, lda]
+// (per = 1: one decay per head; per = D: one per head and key channel).
+__global__ void __launch_bounds__(256) delta_prep_kernel(float *__restrict__ c, int ldc, const float *__restrict__ u, int ldu, int b_col, const float *__restrict__ a, int lda,
+                                                         const float *__restrict__ A_log, const float *__restrict__ dt_bias, float *__restrict__ beta, float *__restrict__ dec,
+                                                         int H, int G, int D, int per) {
+  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  float *cr = c + (size_t)t * ldc;
+  const float qmul = 1.0f / sqrtf((float)D);
+  for (int j = wave; j < 2 * G; j += 4) {  // head j of q | k
+    float *v = cr + (size_t)j * D;
+    float s = 0.f;
+    for (int d = lane; d < D; d += 64) s = fmaf(v[d], v[d], s);
+    const float inv = (1.0f / sqrtf(wave_sum(s) + 1e-6f)) * (j < G ? qmul : 1.0f);
+    for (int d = lane; d < D; d += 64) v[d] *= inv;
+  }
+  for (int h = threadIdx.x; h < H; h += 256) beta[(size_t)t * H + h] = sigmoid_f(u[(size_t)t * ldu + b_col + h]);
+  const int ndec = H * per;
+  for (int e = threadIdx.x; e < ndec; e += 256)
+    dec[(size_t)t * ndec + e] = expf(-expf(A_log[e / per]) * softplus_f(a[(size_t)t * lda + e] + dt_bias[e]));
+}
+
+// ---------------------------------------------------------------------------------- delta rule: the recurrence
+// The value columns of S are independent: lane (p, r) of a wave owns the rows n in [r K, r K + K) of column p, the two sums over n (S^T k before the write, S^T q after it)
+// close with R-lane butterflies.  The waves of one (entry, head) share the rows' operands through LDS: TC rows are staged at a time with coalesced loads, the next TC rows
+// are in registers while the current ones are consumed.  An entry's rows run in order (the write depends on the state), entries / heads / columns in parallel.
+struct DeltaArgs {
+  const float *c;      // [rows, ldc]: q [G * D] | k [G * D] | v [H * Dv]
+  const float *beta;   // [rows, H]
+  const float *dec;    // [rows, H * per]
+  float *state;        // [slots, H, D, Dv]
+  float *out;          // [rows, H * Dv]
+  const int *seq_start, *seq_pos0, *seq_slot;
+  int ldc, H, G, D, Dv, per;
+};
+template <int R, int K, bool VEC, int TC, int MAXC> __global__ void __launch_bounds__(512) delta_scan_kernel(DeltaArgs a, int rowpad) {
+  extern __shared__ __attribute__((aligned(16))) float sm[];  // [2][TC][rowpad]: k [D] | q [D] | decay [per] (padded to 4) | v [Dv] | beta
+  constexpr int PT = 64 / R;
+  const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, r = lane % R, p = (blockIdx.x * (nthr >> 6) + wave) * PT + lane / R;
+  const int h = blockIdx.y, s = blockIdx.z;
+  const int r0 = a.seq_start[s], len = a.seq_start[s + 1] - r0;
+  if (len <= 0) return;
+  const int D = a.D, Dv = a.Dv, per = a.per, g = h / (a.H / a.G);
+  const bool live = p < Dv;
+  const int pc = live ? p : Dv - 1;
+  int nk = D - r * K;
+  nk = nk < 0 ? 0 : (nk > K ? K : nk);
+  float *st = a.state + ((size_t)a.seq_slot[s] * a.H + h) * D * Dv;
+  const bool carried = a.seq_pos0[s] > 0;
+  float S[K];
+#pragma unroll
+  for (int k = 0; k < K; ++k) S[k] = (k < nk && carried) ? st[(size_t)(r * K + k) * Dv + pc] : 0.f;
+  const int perp = (per + 3) & ~3, o_q = D, o_g = 2 * D, o_v = 2 * D + perp, o_b = o_v + Dv, rowlen = o_b + 1, stage = TC * rowpad;
+  const int qcol = g * D, kcol = a.G * D + g * D, vcol = 2 * a.G * D + h * Dv;
+  float stg[TC][MAXC];
+  auto fetch = [&](int c0) {
+#pragma unroll
+    for (int i = 0; i < TC; ++i)
+#pragma unroll
+      for (int m = 0; m < MAXC; ++m) {
+        const int j = tid + m * nthr, row = r0 + c0 + i;
+        float v = 0.f;
+        if (c0 + i < len && j < rowlen) {
+          const float *cr = a.c + (size_t)row * a.ldc;
+          if (j < o_q) v = cr[kcol + j];
+          else if (j < o_g) v = cr[qcol + j - o_q];
+          else if (j < o_v) v = j - o_g < per ? a.dec[((size_t)row * a.H + h) * per + j - o_g] : 0.f;
+          else if (j < o_b) v = cr[vcol + j - o_v];
+          else v = a.beta[(size_t)row * a.H + h];
+        }
+        stg[i][m] = v;
+      }
+  };
+  auto put = [&](float *buf) {
+#pragma unroll
+    for (int i = 0; i < TC; ++i)
+#pragma unroll
+      for (int m = 0; m < MAXC; ++m) {
+        const int j = tid + m * nthr;
+        if (j < rowpad) buf[i * rowpad + j] = stg[i][m];
+      }
+  };
+  fetch(0);
+  put(sm);
+  __syncthreads();
+  int flip = 0;
+  for (int c0 = 0; c0 < len; c0 += TC, flip ^= 1) {
+    const float *cur = sm + flip * stage;
+    const bool more = c0 + TC < len;
+    if (more) fetch(c0 + TC);
+    const int cnt = len - c0 < TC ? len - c0 : TC;
+    for (int i = 0; i < cnt; ++i) {
+      const float *row = cur + i * rowpad;
+      const float vp = row[o_v + pc], be = row[o_b], g1 = row[o_g];
+      const int base = nk ? r * K : 0;
+      float acc = 0.f;
+      if (VEC) {
+#pragma unroll
+        for (int k = 0; k < K; k += 4) {
+          const int kk = base + (k < nk ? k : 0);
+          const float4 k4 = *(const float4 *)(row + kk);
+          float4 g4 = make_float4(g1, g1, g1, g1);
+          if (per > 1) g4 = *(const float4 *)(row + o_g + kk);
+          const bool on = k < nk;
+          const float kv[4] = {on ? k4.x : 0.f, on ? k4.y : 0.f, on ? k4.z : 0.f, on ? k4.w : 0.f}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            S[k + q] *= gv[q];
+            acc = fmaf(S[k + q], kv[q], acc);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          const int kk = k < nk ? base + k : 0;
+          const float kv = k < nk ? row[kk] : 0.f, gv = per > 1 ? row[o_g + kk] : g1;
+          S[k] *= gv;
+          acc = fmaf(S[k], kv, acc);
+        }
+      }
+#pragma unroll
+      for (int m = 1; m < R; m <<= 1) acc += __shfl_xor(acc, m, 64);
+      const float uw = be * (vp - acc);
+      float o = 0.f;
+      if (VEC) {
+#pragma unroll
+        for (int k = 0; k < K; k += 4) {
+          const int kk = base + (k < nk ? k : 0);
+          const float4 k4 = *(const float4 *)(row + kk), q4 = *(const float4 *)(row + o_q + kk);
+          const bool on = k < nk;
+          const float kv[4] = {on ? k4.x : 0.f, on ? k4.y : 0.f, on ? k4.z : 0.f, on ? k4.w : 0.f}, qv[4] = {on ? q4.x : 0.f, on ? q4.y : 0.f, on ? q4.z : 0.f, on ? q4.w : 0.f};
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            S[k + q] = fmaf(kv[q], uw, S[k + q]);
+            o = fmaf(S[k + q], qv[q], o);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          const int kk = k < nk ? base + k : 0;
+          const float kv = k < nk ? row[kk] : 0.f, qv = k < nk ? row[o_q + kk] : 0.f;
+          S[k] = fmaf(kv, uw, S[k]);
+          o = fmaf(S[k], qv, o);
+        }
+      }
+#pragma unroll
+      for (int m = 1; m < R; m <<= 1) o += __shfl_xor(o, m, 64);
+      if (r == 0 && live) a.out[(size_t)(r0 + c0 + i) * a.H * Dv + (size_t)h * Dv + p] = o;
+    }
+    if (more) put(sm + (flip ^ 1) * stage);
+    __syncthreads();
+  }
+  if (live)
+#pragma unroll
+    for (int k = 0; k < K; ++k)
+      if (k < nk) st[(size_t)(r * K + k) * Dv + p] = S[k];
+}
+
+// ---------------------------------------------------------------------------------- exponential gates with a running stabiliser
+// u [rows, ldu]: raw input-gate logits at i_col + h, forget-gate logits at f_col + h, queries [H * D] at q_col (multiplied by q_mult in place).
+//   i = cap tanh((raw_i + bi) / cap);  f = logsigmoid(cap tanh((raw_f + bf) / cap));  m' = max(f + m, i)   (m carried per slot and head, 0 for a fresh sequence)
+//   steps [rows, H, 2] = (e^{i - m'}, e^{f + m - m'}): what the state takes in and what it keeps;  mexp [rows, H] = e^{-m'}
+// One workgroup per entry: the log gates of all its rows in parallel, then the maximum chain (one thread per head, two operations per row), then the exponentials in parallel.
+__global__ void __launch_bounds__(256) exp_gates_kernel(float *__restrict__ u, int ldu, int i_col, int f_col, int q_col, int nq, float q_mult, const float *__restrict__ bi,
+                                                        const float *__restrict__ bf, float cap, float *__restrict__ m_state, float *__restrict__ steps, float *__restrict__ mbuf,
+                                                        float *__restrict__ mexp, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
+                                                        const int *__restrict__ seq_slot, int H) {
+  const int s = blockIdx.x, r0 = seq_start[s], len = seq_start[s + 1] - r0;
+  if (len <= 0) return;
+  for (int e = threadIdx.x; e < len * H; e += 256) {
+    const int t = r0 + e / H, h = e % H;
+    const float *ur = u + (size_t)t * ldu;
+    const float ig = cap * tanhf((ur[i_col + h] + bi[h]) / cap), fr = cap * tanhf((ur[f_col + h] + bf[h]) / cap);
+    steps[2 * ((size_t)t * H + h)] = ig;
+    steps[2 * ((size_t)t * H + h) + 1] = -softplus_f(-fr);
+  }
+  if (q_mult != 1.0f)
+    for (size_t e = threadIdx.x; e < (size_t)len * nq; e += 256) u[(size_t)(r0 + e / nq) * ldu + q_col + e % nq] *= q_mult;
+  __syncthreads();
+  float *ms = m_state + (size_t)seq_slot[s] * H;
+  const bool carried = seq_pos0[s] > 0;
+  if (threadIdx.x < H) {
+    const int h = threadIdx.x;
+    float m = carried ? ms[h] : 0.f;
+    for (int i = 0; i < len; ++i) {
+      const float *g = steps + 2 * ((size_t)(r0 + i) * H + h);
+      m = fmaxf(g[1] + m, g[0]);
+      mbuf[(size_t)(r0 + i) * H + h] = m;
+    }
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < len * H; e += 256) {
+    const int i = e / H, h = e % H, t = r0 + i;
+    const float m_old = i ? mbuf[(size_t)(t - 1) * H + h] : (carried ? ms[h] : 0.f), m_new = mbuf[(size_t)t * H + h];
+    float *g = steps + 2 * ((size_t)t * H + h);
+    const float ig = g[0], fg = g[1];
+    g[0] = expf(ig - m_new);
+    g[1] = expf(fg + m_old - m_new);
+    mexp[(size_t)t * H + h] = expf(-m_new);
+  }
+  __syncthreads();   // every m_old has been read
+  if (threadIdx.x < H) ms[threadIdx.x] = mbuf[(size_t)(r0 + len - 1) * H + threadIdx.x];
+}
+
+// ---------------------------------------------------------------------------------- per-head output norm with a gate
+// y [rows, H * ldp] f32 (head h's Dv values start at h * ldp).  mexp (nullable, [rows, H]): the values are first divided by max(|y[h * ldp + Dv]|, mexp) + 1e-6 (the
+// normaliser column of a matrix memory).  Then o / sqrt(mean(o^2) + eps) times w (w_full: [H * Dv], else [Dv] shared by the heads) times the gate: gate_mode 1 = sigmoid,
+// 2 = SiLU of gate[t * ldg + h * Dv + d]; 0 = none.  One wave per (row, head).
+template <class T> __global__ void __launch_bounds__(64) head_norm_gate_kernel(const float *__restrict__ y, int ldp, const float *__restrict__ mexp, const float *__restrict__ w,
+                                                                               int w_full, const float *__restrict__ gate, int ldg, int gate_mode, T *__restrict__ out, int H, int Dv,
+                                                                               float eps) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const float *yr = y + ((size_t)t * H + h) * ldp;
+  float den = 1.0f;
+  if (mexp) den = 1.0f / (fmaxf(fabsf(yr[Dv]), mexp[(size_t)t * H + h]) + 1e-6f);
+  float s = 0.f;
+  for (int d = lane; d < Dv; d += 64) {
+    const float v = mexp ? yr[d] * den : yr[d];
+    s = fmaf(v, v, s);
+  }
+  const float inv = 1.0f / sqrtf(wave_sum(s) / (float)Dv + eps);
+  for (int d = lane; d < Dv; d += 64) {
+    float v = (mexp ? yr[d] * den : yr[d]) * inv * w[(w_full ? h * Dv : 0) + d];
+    if (gate_mode) {
+      const float gv = gate[(size_t)t * ldg + (size_t)h * Dv + d];
+      v *= gate_mode == 1 ? sigmoid_f(gv) : silu_f(gv);
+    }
+    out[((size_t)t * H + h) * Dv + d] = from_f<T>(v);
+  }
+}
+
+// ---------------------------------------------------------------------------------- x (+)= c (y1 / rms(y1) w1 + y2 / rms(y2) w2)
+__global__ void __launch_bounds__(256) norm_pair_add_kernel(float *__restrict__ x, int ldx, const float *__restrict__ y1, const float *__restrict__ w1, const float *__restrict__ y2,
+                                                            const float *__restrict__ w2, int W, float eps, float c, int accumulate) {
+  __shared__ float red[4];
+  const int t = blockIdx.x;
+  const float *a = y1 + (size_t)t * W, *b = y2 + (size_t)t * W;
+  float s1 = 0.f, s2 = 0.f;
+  for (int k = threadIdx.x; k < W; k += 256) { s1 = fmaf(a[k], a[k], s1); s2 = fmaf(b[k], b[k], s2); }
+  const float i1 = 1.0f / sqrtf(block_sum_256(s1, red) / (float)W + eps);
+  const float i2 = 1.0f / sqrtf(block_sum_256(s2, red) / (float)W + eps);
+  for (int k = threadIdx.x; k < W; k += 256) {
+    const float v = c * (a[k] * i1 * w1[k] + b[k] * i2 * w2[k]);
+    float *xp = x + (size_t)t * ldx + k;
+    *xp = accumulate ? *xp + v : v;
+  }
+}
+
+// out [rows, n] (T, contiguous) = the first n columns of u [rows, ldu], rounded once: a column block of a product's f32 result as the operand of the next product
+template <class T> __global__ void __launch_bounds__(256) round_cols_kernel(const float *__restrict__ u, int ldu, T *__restrict__ out, int n, size_t total) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  out[i] = from_f<T>(u[(i / n) * ldu + i % n]);
+}
+
+template <class T> __global__ void __launch_bounds__(256) relu_sq_kernel(const float *__restrict__ u, T *__restrict__ out, size_t n) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const float v = fmaxf(u[i], 0.f);
+  out[i] = from_f<T>(v * v);
+}
+
+}  // namespace hybr
+}  // namespace mrs
+
+using namespace mrs::hybr;
+#define S_(s) ((hipStream_t)(s))
+
+extern "C" const char *mrs_hyb_recur_last_error() { return g_err; }
+
+/* out1 = x / rms(x) * w1, out2 = x / rms(x) * w2 (one_plus: 1 + w) in dtype; out2_32 (nullable): the second one in f32 too */
+extern "C" int mrs_hyb_rmsnorm_pair(const float *x, int ldx, const float *w1, const float *w2, void *out1, void *out2, float *out2_32, int rows, int W, float eps, int one_plus,
+                                    int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (dtype == 1) hipLaunchKernelGGL(rmsnorm_pair_kernel<mrs::bf16_t>, dim3(rows), dim3(256), 0, S_(stream), x, ldx, w1, w2, (mrs::bf16_t *)out1, (mrs::bf16_t *)out2, out2_32, W, eps, one_plus);
+  else if (dtype == 2) hipLaunchKernelGGL(rmsnorm_pair_kernel<float>, dim3(rows), dim3(256), 0, S_(stream), x, ldx, w1, w2, (float *)out1, (float *)out2, out2_32, W, eps, one_plus);
+  else return fail("mrs_hyb_rmsnorm_pair: dtype");
+  return ok_or("mrs_hyb_rmsnorm_pair");
+}
+
+extern "C" int mrs_hyb_delta_prep(float *c, int ldc, const float *u, int ldu, int b_col, const float *a, int lda, const float *A_log, const float *dt_bias, float *beta, float *dec,
+                                  int rows, int H, int G, int D, int per, void *stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || (per != 1 && per != D)) return fail("mrs_hyb_delta_prep: head sizes (heads % kv_heads == 0; decays per head or per key channel)");
+  hipLaunchKernelGGL(delta_prep_kernel, dim3(rows), dim3(256), 0, S_(stream), c, ldc, u, ldu, b_col, a, lda, A_log, dt_bias, beta, dec, H, G, D, per);
+  return ok_or("mrs_hyb_delta_prep");
+}
+
+/* c [rows, ldc] = q [G * D] | k [G * D] | v [H * Dv] (unit q / k), beta [rows, H], dec [rows, H * per] (per 1 or D), state [slots, H, D, Dv], out [rows, H * Dv].
+ * lanes_per_column 0: chosen from the step's parallelism (4 when entries x heads x columns fill the chip, else 16: shorter serial chains). */
+extern "C" int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, const float *dec, float *state, float *out, const int *seq_start, const int *seq_pos0,
+                                  const int *seq_slot, int rows, int entries, int H, int G, int D, int Dv, int per, int lanes_per_column, void *stream) {
+  if (rows <= 0 || entries <= 0) return 0;
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || (per != 1 && per != D)) return fail("mrs_hyb_delta_scan: head sizes (heads % kv_heads == 0; decays per head or per key channel)");
+  if (D > 256) return fail("mrs_hyb_delta_scan: key size above 256");
+  if (entries > 65535 || H > 65535) return fail("mrs_hyb_delta_scan: more than 65535 entries or heads");
+  if (ldc < 2 * G * D + H * Dv) return fail("mrs_hyb_delta_scan: rows shorter than q | k | v");
+  DeltaArgs a{c, beta, dec, state, out, seq_start, seq_pos0, seq_slot, ldc, H, G, D, Dv, per};
+  int R = lanes_per_column;
+  if (R != 4 && R != 16) R = ((long long)entries * H * ((Dv + 15) / 16) >= 1024 || D < 64) ? 4 : 16;
+  const int PT = 64 / R;
+  const int nw_all = (Dv + PT - 1) / PT, nw = nw_all > 8 ? 8 : nw_all, nblk = (nw_all + nw - 1) / nw;
+  const int perp = (per + 3) & ~3, rowlen = 2 * D + perp + Dv + 1, rowpad = (rowlen + 3) & ~3;
+  constexpr int TC = 4, MAXC = 8;
+  if (rowpad > MAXC * 64 * nw) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers (key size far above value size)");
+  const size_t lds = (size_t)2 * TC * rowpad * 4;
+  if (lds > 65536) return fail("mrs_hyb_delta_scan: staged rows above 64 KB");
+  const bool vec = D % 4 == 0;
+  dim3 grid(nblk, H, entries), block(64 * nw);
+#define MRS_DELTA_(R_, K_, V_) hipLaunchKernelGGL((delta_scan_kernel<R_, K_, V_, TC, MAXC>), grid, block, lds, S_(stream), a, rowpad)
+#define MRS_DELTA(R_, K_) do { if (vec) MRS_DELTA_(R_, K_, true); else MRS_DELTA_(R_, K_, false); } while (0)
+  if (R == 4) {
+    if (D <= 32) MRS_DELTA(4, 8); else if (D <= 64) MRS_DELTA(4, 16); else if (D <= 128) MRS_DELTA(4, 32); else MRS_DELTA(4, 64);
+  } else {
+    if (D <= 64) MRS_DELTA(16, 4); else if (D <= 128) MRS_DELTA(16, 8); else MRS_DELTA(16, 16);
+  }
+#undef MRS_DELTA
+#undef MRS_DELTA_
+  return ok_or("mrs_hyb_delta_scan");
+}
+
+/* steps [rows, H, 2], mbuf [rows, H] (scratch), mexp [rows, H]; m_state [slots, H]; the query columns of u are multiplied by q_mult in place */
+extern "C" int mrs_hyb_exp_gates(float *u, int ldu, int i_col, int f_col, int q_col, int nq, float q_mult, const float *bi, const float *bf, float cap, float *m_state,
+                                 float *steps, float *mbuf, float *mexp, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, void *stream) {
+  if (rows <= 0 || entries <= 0) return 0;
+  if (H <= 0 || H > 256 || !(cap > 0.f)) return fail("mrs_hyb_exp_gates: 1 .. 256 heads, a positive gate cap");
+  hipLaunchKernelGGL(exp_gates_kernel, dim3(entries), dim3(256), 0, S_(stream), u, ldu, i_col, f_col, q_col, nq, q_mult, bi, bf, cap, m_state, steps, mbuf, mexp, seq_start,
+                     seq_pos0, seq_slot, H);
+  return ok_or("mrs_hyb_exp_gates");
+}
+
+extern "C" int mrs_hyb_head_norm_gate(const float *y, int ldp, const float *mexp, const float *w, int w_full, const float *gate, int ldg, int gate_mode, void *out, int rows,
+                                      int H, int Dv, float eps, int dtype, void *stream) {
+  if (rows <= 0) return 0;
+  if (H <= 0 || H > 65535 || Dv <= 0 || ldp < Dv + (mexp ? 1 : 0) || gate_mode < 0 || gate_mode > 2 || (gate_mode && !gate)) return fail("mrs_hyb_head_norm_gate: head sizes / gate mode");
+  if (dtype == 1) hipLaunchKernelGGL(head_norm_gate_kernel<mrs::bf16_t>, dim3(rows, H), dim3(64), 0, S_(stream), y, ldp, mexp, w, w_full, gate, ldg, gate_mode, (mrs::bf16_t *)out, H, Dv, eps);
+  else if (dtype == 2) hipLaunchKernelGGL(head_norm_gate_kernel<float>, dim3(rows, H), dim3(64), 0, S_(stream), y, ldp, mexp, w, w_full, gate, ldg, gate_mode, (float *)out, H, Dv, eps);
+  else return fail("mrs_hyb_head_norm_gate: dtype");
+  return ok_or("mrs_hyb_head_norm_gate");
+}
+
+extern "C" int mrs_hyb_norm_pair_add(float *x, int ldx, const float *y1, const float *w1, const float *y2, const float *w2, int rows, int W, float eps, float c, int accumulate,
+                                     void *stream) {
+  if (rows <= 0) return 0;
+  hipLaunchKernelGGL(norm_pair_add_kernel, dim3(rows), dim3(256), 0, S_(stream), x, ldx, y1, w1, y2, w2, W, eps, c, accumulate);
+  return ok_or("mrs_hyb_norm_pair_add");
+}
+
+extern "C" int mrs_hyb_round_cols(const float *u, int ldu, void *out, int rows, int n, int dtype, void *stream) {
+  const size_t total = (size_t)rows * n;
+  if (total == 0) return 0;
+  dim3 grid((unsigned)((total + 255) / 256));
+  if (dtype == 1) hipLaunchKernelGGL(round_cols_kernel<mrs::bf16_t>, grid, dim3(256), 0, S_(stream), u, ldu, (mrs::bf16_t *)out, n, total);
+  else if (dtype == 2) hipLaunchKernelGGL(round_cols_kernel<float>, grid, dim3(256), 0, S_(stream), u, ldu, (float *)out, n, total);
+  else return fail("mrs_hyb_round_cols: dtype");
+  return ok_or("mrs_hyb_round_cols");
+}
+
+extern "C" int mrs_hyb_relu_sq(const float *u, void *out, int rows, int ff, int dtype, void *stream) {
+  const size_t n = (size_t)rows * ff;
+  if (n == 0) return 0;
+  dim3 grid((unsigned)((n + 255) / 256));
+  if (dtype == 1) hipLaunchKernelGGL(relu_sq_kernel<mrs::bf16_t>, grid, dim3(256), 0, S_(stream), u, (mrs::bf16_t *)out, n);
+  else if (dtype == 2) hipLaunchKernelGGL(relu_sq_kernel<float>, grid, dim3(256), 0, S_(stream), u, (float *)out, n);
+  else return fail("mrs_hyb_relu_sq: dtype");
+  return ok_or("mrs_hyb_relu_sq");
+}

@@ -59,10 +59,24 @@ _SIGS = {
     "mrs_hyb_layernorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     "mrs_hyb_qkv_bias_temp_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp],
     "mrs_hyb_paged_talk_sigmoid_attn": [_vp] * 9 + [_i, _vp] + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp, _i, _vp],
+    "mrs_hyb_gated_scan": [_vp, _i] + [_vp] * 11 + [_i] * 8 + [_vp],
+    "mrs_hyb_qk_headnorm_rope_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
+    "mrs_hyb_paged_attn_chunked": [_vp] * 7 + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _vp, _i, _i, _vp, _i, _vp],
+    "mrs_hyb_route_topk_softmax": [_vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _vp],
+    "mrs_hyb_rmsnorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
+    "mrs_hyb_delta_prep": [_vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "mrs_hyb_delta_scan": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 8 + [_vp],
+    "mrs_hyb_exp_gates": [_vp, _i, _i, _i, _i, _i, _f, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "mrs_hyb_head_norm_gate": [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _vp],
+    "mrs_hyb_norm_pair_add": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _i, _vp],
+    "mrs_hyb_round_cols": [_vp, _i, _vp, _i, _i, _i, _vp],
+    "mrs_hyb_relu_sq": [_vp, _vp, _i, _i, _i, _vp],
     "mrs_hyb_gemm": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _i, _l, _i, _vp],
     "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp],
     "mrs_hyb_gemv_act": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp, _f, _f, _vp],
 }
+_RECUR = {"mrs_hyb_rmsnorm_pair", "mrs_hyb_delta_prep", "mrs_hyb_delta_scan", "mrs_hyb_exp_gates", "mrs_hyb_head_norm_gate", "mrs_hyb_norm_pair_add", "mrs_hyb_round_cols",
+          "mrs_hyb_relu_sq"}   # launchers of csrc/hyb_recur.hip (their own error text)
 _fns: dict = {}
 _step_stream: Optional[int] = None   # the stream handle of the step in progress (looked up once per forward_batch, not once per launch)
 
@@ -74,7 +88,7 @@ def _call(name: str, *args) -> None:
         fn = _fns[name] = _lib.sym("hybrid", name, _SIGS[name], C.c_int)
     conv = [a.data_ptr() if isinstance(a, torch.Tensor) else a for a in args]
     if fn(*conv, _step_stream if _step_stream is not None else torch.cuda.current_stream().cuda_stream) != 0:
-        err = _lib.sym("hybrid", "mrs_hyb_gemm_last_error" if "gem" in name else ("mrs_hyb_talk_last_error" if "talk" in name else "mrs_hyb_last_error"), [], C.c_char_p)()
+        err = _lib.sym("hybrid", "mrs_hyb_recur_last_error" if name in _RECUR else "mrs_hyb_gemm_last_error" if "gem" in name else ("mrs_hyb_talk_last_error" if "talk" in name else "mrs_hyb_last_error"), [], C.c_char_p)()
         raise ValueError((err or b"").decode() or name)
 
 
@@ -213,6 +227,42 @@ class AttentionSpec:
     keep_first: int = 0        # tokens at the start of the sequence that stay visible behind the window
     rotary: Optional[RotarySpec] = None
     qk_norm: bool = True       # plain-weight RMS norm over the whole query / key projection, before rotation
+    chunk: int = 0             # > 0: position i sees j <= i only when floor(i / chunk) == floor(j / chunk) (chunks counted from position 0; excludes `window`)
+    head_norm: bool = False    # the query / key norm runs per head with weights [dim] shared by the heads
+    sink: bool = False         # the softmax's denominator has one more term e^{sink_h}, a learned number per head (tensor `sink`)
+    head_gate: bool = False    # head h's output is multiplied by sigmoid(Wg h)_h, one logit per head (tensor `g` [heads, width])
+
+
+@dataclass
+class DeltaRuleSpec:
+    """Gated delta rule (DeltaRuleMixer): S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.  `decay`: "head" = one decay per head from the projection `a`,
+    "channel" = one per head and key channel from the two-step projection `a1`, `a2`.  `gate`: "silu" = SiLU of the full projection `g`, "sigmoid_lowrank" = sigmoid of the
+    two-step projection `g1`, `g2` (the inner sizes of both two-step projections come from the tensors)."""
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    decay: str = "head"
+    gate: str = "silu"
+
+
+@dataclass
+class MlstmSpec:
+    """Matrix memory with exponential input / forget gates and a running stabiliser (MlstmMixer)."""
+    heads: int
+    dim: int
+    vdim: int
+    gate_cap: float
+
+
+@dataclass
+class ParallelSpec:
+    """Two mixers side by side on the same input; the result is half the sum of their outputs, each normed over the model width (ParallelMixer)."""
+    left_kind: str
+    left: object
+    right_kind: str
+    right: object
 
 
 @dataclass
@@ -306,6 +356,16 @@ class ClampedMoeSpec:
 
 
 @dataclass
+class TopkSoftmaxMoeSpec:
+    """Routed squared-ReLU experts without gates; the weights are a softmax over the chosen logits (TopkSoftmaxReluSqMoe)."""
+    experts: int
+    top: int
+    ff: int
+    shared_ff: int = 0
+    kind = "moe_topk_softmax_relu2"
+
+
+@dataclass
 class DenseSpec:
     """down(xIELU(up h + b) ) + b (XieluFeedForward)."""
     ff: int
@@ -325,6 +385,7 @@ class LayerSpec:
     mixer: object
     ff: Optional[object]       # MoeSpec | ClampedMoeSpec | DenseSpec | None
     prefix: str                # tensor-name prefix of the layer
+    weights_of: Optional[int] = None   # index of the layer whose tensors (mixer, feed-forward, norms) this layer uses; its pages and state slots are its own
 
 
 @dataclass
@@ -336,7 +397,8 @@ class HybridSpec:
     embed: str = "embed"
     final_norm: str = "final.norm"
     head: str = "head"
-    norm: str = "rms_one_plus"   # "rms_one_plus": x / rms * (1 + w);  "layer": (x - mean) / sqrt(var + eps) * w + b, the bias being the tensor `<name>.b`
+    norm: str = "rms_one_plus"   # "rms_one_plus": x / rms * (1 + w);  "rms": x / rms * w;  "layer": (x - mean) / sqrt(var + eps) * w + b, the bias being the tensor `<name>.b`
+    parallel_sublayers: bool = False   # x += mixer(norm1(x)) + feed_forward(norm2(x)), both norms of the same x (else one sublayer after the other)
     post_norms: bool = False     # every sublayer's output is normed (`norm1b` / `norm2b`) before it joins the residual stream
     embed_norm: Optional[str] = None   # tensor of a norm (of the model's kind) applied to the embedding rows
     residual_mult: float = 1.0   # every sublayer's output is multiplied by this before it joins the residual stream(s)
@@ -448,6 +510,50 @@ def setopel_spec(cfg: dict) -> HybridSpec:
                       streams=int(cfg.get("streams", 0) or 0))
 
 
+def gifopel_spec(cfg: dict) -> HybridSpec:
+    """config.json of a Gifopel checkpoint -> the layer list: plain-weight RMS norms, layers whose mixer and feed-forward read two norms of the same residual row, mixers
+    `channel_delta` (delta rule with decays per key channel), `mlstm`, `parallel` (chunked sink attention next to a delta rule with decays per head), dense SiLU-GLU or routed
+    squared-ReLU feed-forwards, layers that use another layer's tensors, a head tied to the embedding.  Every size and every model-dependent constant comes from the file."""
+    def delta(m, decay, gate):
+        return DeltaRuleSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m["vdim"]), int(m["conv"]), decay, gate)
+
+    def attention(m):
+        rot, mask = m.get("rot"), m.get("mask") or {}
+        return AttentionSpec(int(m["heads"]), int(m.get("kv_heads", m["heads"])), int(m["dim"]), int(m["vdim"]), float(m["scale"]), 0, 0,
+                             RotarySpec(int(rot["dims"]), float(rot["base"])) if rot and int(rot.get("dims", 0)) > 0 else None, True,
+                             chunk=int(mask.get("size", 0) or 0), head_norm=True, sink=True, head_gate=True)
+    layers = []
+    for i, L in enumerate(cfg["layers"]):
+        m, kind = L["mixer"], L["type"]
+        if kind == "channel_delta":
+            kind, mixer = "delta_rule", delta(m, "channel", "sigmoid_lowrank")
+        elif kind == "mlstm":
+            mixer = MlstmSpec(int(m["heads"]), int(m["dim"]), int(m["vdim"]), float(m["gate_cap"]))
+        elif kind == "parallel":
+            mixer = ParallelSpec("attention", attention(m["left"]), "delta_rule", delta(m["right"], "head", "silu"))
+        else:
+            raise ValueError(f"Gifopel: unknown layer type {L['type']!r}")
+        f = L.get("mlp")
+        ff = None
+        if f:
+            if f.get("kind") == "dense":
+                ff = GluSpec(int(f["ff"]))
+            elif f.get("kind") == "moe":
+                ff = TopkSoftmaxMoeSpec(int(f["router"]["experts"]), int(f["router"]["top"]), int(f["expert"]["ff"]))
+            else:
+                raise ValueError(f"Gifopel: unknown feed-forward kind {f.get('kind')!r}")
+        src = L.get("weights_of")
+        layers.append(LayerSpec(kind, mixer, ff, f"l{i if src is None else int(src)}.", None if src is None else int(src)))
+    for i, ls in enumerate(layers):
+        j = ls.weights_of
+        if j is not None:
+            if not 0 <= j < len(layers) or j == i or layers[j].weights_of is not None:
+                raise ValueError(f"Gifopel: layer {i} uses the tensors of layer {j}, which has none of its own")
+            if (layers[j].kind, layers[j].mixer, layers[j].ff) != (ls.kind, ls.mixer, ls.ff):
+                raise ValueError(f"Gifopel: layer {i} uses the tensors of layer {j} but is described differently")
+    return HybridSpec(int(cfg["vocab"]), int(cfg["width"]), float(cfg["norm"]["eps"]), layers, head="embed", norm="rms", parallel_sublayers=True)
+
+
 # ------------------------------------------------------------------------------------------------------------------ mixers and feed-forwards
 class _Module:
     out_bias = None            # f32 bias of the module's last product, left to the caller (a norm that follows adds it while it reads the product)
@@ -460,6 +566,16 @@ class _Module:
         """A checkpoint tensor on the device: GEMM operands in the serving dtype, everything else f32."""
         t = get(name)
         return t.to(self.m.device, self.m.torch_dtype if gemm else torch.float32).contiguous()
+
+    def carried(self):
+        return ()
+
+    def share_from(self, other: "_Module") -> None:
+        """Use `other`'s loaded tensors (a layer that borrows another layer's weights); what this module carries per sequence -- pages, taps, states -- stays its own."""
+        mine = {k for k, v in self.__dict__.items() if isinstance(v, torch.Tensor) and any(v is t for t in self.carried())}
+        for k, v in other.__dict__.items():
+            if k not in mine and k != "m":
+                setattr(self, k, v)
 
 
 class Mamba2Mixer(_Module):
@@ -527,10 +643,23 @@ class WindowAttention(_Module):
         q, k, v = (get(p + n) for n in ("q", "k", "v"))
         if q.shape[0] != s.heads * s.dim or k.shape[0] != s.kv_heads * s.dim or v.shape[0] != s.kv_heads * s.vdim:
             raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
-        self.w_qkv = torch.cat([q, k, v], 0).to(self.m.device, self.m.torch_dtype).contiguous()
+        parts = [q, k, v]
+        if s.head_gate:
+            parts.append(get(p + "g"))
+            if tuple(parts[-1].shape) != (s.heads, q.shape[1]):
+                raise ValueError(f"{p}: the gate projection has one row per head")
+        self.w_qkv = torch.cat(parts, 0).to(self.m.device, self.m.torch_dtype).contiguous()   # [q | k | v (| gate logits), W]
+        self.gate_col = s.heads * s.dim + s.kv_heads * (s.dim + s.vdim)
         self.w_o = self.w(get, p + "o", True)
         self.q_norm = self.w(get, p + "q.norm", False) if s.qk_norm else None
         self.k_norm = self.w(get, p + "k.norm", False) if s.qk_norm else None
+        if s.qk_norm and (self.q_norm.numel(), self.k_norm.numel()) != ((s.dim, s.dim) if s.head_norm else (s.heads * s.dim, s.kv_heads * s.dim)):
+            raise ValueError(f"{p}: query / key norm weights do not match the mixer's sizes")
+        self.sink = self.w(get, p + "sink", False) if s.sink else None
+        if s.sink and self.sink.numel() != s.heads:
+            raise ValueError(f"{p}: one sink per head")
+        if s.chunk and (s.window or s.keep_first):
+            raise ValueError(f"{p}: chunks and a sliding window exclude each other")
 
     def carried(self):
         return (self.k_cache, self.v_cache)
@@ -543,11 +672,20 @@ class WindowAttention(_Module):
         T = b.rows
         qkv = m.linear(h, self.w_qkv)
         q = torch.empty(T, s.heads * s.dim, dtype=m.torch_dtype, device=m.device)
-        _call("mrs_hyb_qk_norm_rope_cache", qkv, qkv.stride(0), self.q_norm, self.k_norm, self.freq, b.tok_pos, b.slot_mapping, q, self.k_cache, self.v_cache, T,
-              s.heads, s.kv_heads, s.dim, s.vdim, s.rotary.dims if s.rotary else 0, m.block_size, m.spec.eps, m.dt)
+        _call("mrs_hyb_qk_headnorm_rope_cache" if s.head_norm else "mrs_hyb_qk_norm_rope_cache", qkv, qkv.stride(0), self.q_norm, self.k_norm, self.freq, b.tok_pos,
+              b.slot_mapping, q, self.k_cache, self.v_cache, T, s.heads, s.kv_heads, s.dim, s.vdim, s.rotary.dims if s.rotary else 0, m.block_size, m.spec.eps, m.dt)
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=m.device)
-        _call("mrs_hyb_paged_window_attn", q, self.k_cache, self.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size,
-              b.max_blocks, s.window, s.keep_first, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
+        if s.chunk or s.sink or s.head_gate:
+            if s.window or s.keep_first:
+                raise NotImplementedError("a learned sink / a per-head gate beside a sliding window")
+            # a chunk holds few keys: no key splits (unchunked layers of single-row steps may split)
+            scratch, splits = (None, 0) if s.chunk else m.key_splits(b, s.heads, s.vdim)
+            _call("mrs_hyb_paged_attn_chunked", q, self.k_cache, self.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size,
+                  b.max_blocks, s.chunk, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, int(s.sink), self.sink,
+                  qkv[:, self.gate_col:] if s.head_gate else None, qkv.stride(0), 1, scratch, splits)
+        else:
+            _call("mrs_hyb_paged_window_attn", q, self.k_cache, self.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size,
+                  b.max_blocks, s.window, s.keep_first, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
         m.linear(o, self.w_o, out=x, accumulate=accumulate)
 
 
@@ -988,9 +1126,226 @@ class GluFeedForward(_Module):
         m.linear(a, self.w_down, out=x, accumulate=accumulate)
 
 
-MIXERS: Dict[str, Callable] = {"mamba2": Mamba2Mixer, "attention": WindowAttention, "talk_attention": TalkSigmoidAttention, "sink_attention": GatedSinkAttention,
+class DeltaRuleMixer(_Module):
+    """q, k (kv_heads x dim), v (heads x vdim), the write strengths and the first steps of the decay / gate projections are ONE product; q, k, v pass a short causal
+    convolution + SiLU (taps carried per slot); q and k become unit vectors per head (q times dim^(-1/2)); beta = sigmoid; g = exp(-exp(A_log_h) softplus(a + dt_bias)) per
+    head or per (head, key channel).  Per head the f32 state S [dim, vdim] (carried per slot): S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
+    o / rms(o) per head times the weight `norm` [vdim] times the gate, then the output projection.  Head h reads q / k head h // (heads / kv_heads)."""
+
+    def __init__(self, model, spec: DeltaRuleSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        if spec.heads % spec.kv_heads or spec.decay not in ("head", "channel") or spec.gate not in ("silu", "sigmoid_lowrank") or spec.conv < 1:
+            raise ValueError(f"{prefix}: heads % kv_heads must be 0; decay head | channel; gate silu | sigmoid_lowrank; at least one tap")
+        dev = model.device
+        self.nqk, self.nv = spec.kv_heads * spec.dim, spec.heads * spec.vdim
+        self.channels = 2 * self.nqk + self.nv
+        self.per = spec.dim if spec.decay == "channel" else 1
+        self.conv_state = torch.zeros(model.state_slots, self.channels, max(spec.conv - 1, 1), dtype=torch.float32, device=dev)
+        self.state = torch.zeros(model.state_slots, spec.heads, spec.dim, spec.vdim, dtype=torch.float32, device=dev)
+
+    def carried(self):
+        return (self.conv_state, self.state)
+
+    def state_bytes_per_slot(self) -> int:
+        return 4 * (self.conv_state[0].numel() + self.state[0].numel())
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        dev, dt = self.m.device, self.m.torch_dtype
+        lowrank_a, lowrank_g = s.decay == "channel", s.gate == "sigmoid_lowrank"
+        parts = [get(p + n) for n in ("q", "k", "v", "b", "a1" if lowrank_a else "a", "g1" if lowrank_g else "g")]
+        ndec = s.heads * self.per
+        self.rank_a = parts[4].shape[0] if lowrank_a else 0
+        self.rank_g = parts[5].shape[0] if lowrank_g else 0
+        want = [self.nqk, self.nqk, self.nv, s.heads, self.rank_a or ndec, self.rank_g or self.nv]
+        if [t.shape[0] for t in parts] != want or any(t.shape[1] != W for t in parts):
+            raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
+        self.w_in = torch.cat(parts, 0).to(dev, dt).contiguous()            # [q | k | v | beta | a (a1) | g (g1), W]
+        self.b_col = self.channels
+        self.a_col = self.b_col + s.heads
+        self.g_col = self.a_col + want[4]
+        self.w_a2 = self.w(get, p + "a2", True) if lowrank_a else None
+        self.w_g2 = self.w(get, p + "g2", True) if lowrank_g else None
+        self.conv_w = torch.cat([get(p + n + ".conv") for n in ("q", "k", "v")], 0).to(dev, torch.float32).contiguous()   # [channels, taps]
+        self.A_log, self.dt_bias, self.norm = (self.w(get, p + n, False).reshape(-1) for n in ("A_log", "dt_bias", "norm"))
+        self.w_o = self.w(get, p + "o", True)
+        if tuple(self.conv_w.shape) != (self.channels, s.conv) or self.A_log.numel() != s.heads or self.dt_bias.numel() != ndec or self.norm.numel() != s.vdim or \
+                tuple(self.w_o.shape) != (W, self.nv) or (lowrank_a and tuple(self.w_a2.shape) != (ndec, self.rank_a)) or \
+                (lowrank_g and tuple(self.w_g2.shape) != (self.nv, self.rank_g)):
+            raise ValueError(f"{p}: convolution / decay / gate / output shapes do not match the mixer's sizes")
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T, dev = b.rows, m.device
+        f32 = dict(dtype=torch.float32, device=dev)
+        u = m.linear(h, self.w_in)                                          # f32 [T, q | k | v | beta | a | g]
+        c = torch.empty(T, self.channels, **f32)
+        _call("mrs_hyb_conv", u, u.stride(0), None, self.conv_w, None, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, c, T, b.entries, self.channels,
+              s.conv, 1)
+        a = u[:, self.a_col:]
+        if self.w_a2 is not None:                                           # the decay's second step: a product on the rounded first step
+            a = m.linear(m.round_cols(a, self.rank_a), self.w_a2)
+        gate = u[:, self.g_col:]
+        if self.w_g2 is not None:
+            gate = m.linear(m.round_cols(gate, self.rank_g), self.w_g2)
+        beta = torch.empty(T, s.heads, **f32)
+        dec = torch.empty(T, s.heads * self.per, **f32)
+        _call("mrs_hyb_delta_prep", c, c.stride(0), u, u.stride(0), self.b_col, a, a.stride(0), self.A_log, self.dt_bias, beta, dec, T, s.heads, s.kv_heads, s.dim, self.per)
+        y = torch.empty(T, self.nv, **f32)
+        _call("mrs_hyb_delta_scan", c, c.stride(0), beta, dec, self.state, y, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, s.heads, s.kv_heads, s.dim, s.vdim,
+              self.per, 0)
+        o = torch.empty(T, self.nv, dtype=m.torch_dtype, device=dev)
+        _call("mrs_hyb_head_norm_gate", y, s.vdim, None, self.norm, 0, gate, gate.stride(0), 1 if self.w_g2 is not None else 2, o, T, s.heads, s.vdim, m.spec.eps, m.dt)
+        m.linear(o, self.w_o, out=x, accumulate=accumulate)
+
+
+class MlstmMixer(_Module):
+    """v | k | q | gate | input-gate | forget-gate logits in one product; q times dim^(-1/2); log gates i = cap tanh((.. + b) / cap), f = logsigmoid(cap tanh((.. + b) /
+    cap)); with the running maximum m' = max(f + m, i) (m starts at 0): S <- e^{f + m - m'} S + e^{i - m'} k v^T, n likewise with k alone, o = S^T q / (max(|n . q|,
+    e^{-m'}) + 1e-6).  n rides as one more column of the state (a value that is always 1), so the recurrence is the gated scan of the state-space mixers with step values
+    from the gates: portions run their segments in parallel.  o / rms(o) per head, times `norm` [heads * vdim], times sigmoid(gate), output projection.  Carries S | n
+    [heads, dim, vdim + 1] and m [heads] per slot, f32."""
+
+    def __init__(self, model, spec: MlstmSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        dev = model.device
+        self.state = torch.zeros(model.state_slots, spec.heads, spec.dim, spec.vdim + 1, dtype=torch.float32, device=dev)
+        self.m_state = torch.zeros(model.state_slots, spec.heads, dtype=torch.float32, device=dev)
+        self.q_mult = float(np.float32(spec.dim) ** np.float32(-0.5))
+
+    def carried(self):
+        return (self.state, self.m_state)
+
+    def state_bytes_per_slot(self) -> int:
+        return 4 * (self.state[0].numel() + self.m_state[0].numel())
+
+    def load(self, get):
+        s, p, W = self.s, self.p, self.m.spec.width
+        parts = [get(p + n) for n in ("v", "k", "q", "g", "i", "f")]
+        nv, nk = s.heads * s.vdim, s.heads * s.dim
+        want = [nv, nk, nk, nv, s.heads, s.heads]
+        if [t.shape[0] for t in parts] != want or any(t.shape[1] != W for t in parts):
+            raise ValueError(f"{p}: projection shapes do not match the mixer's sizes")
+        self.w_in = torch.cat(parts, 0).to(self.m.device, self.m.torch_dtype).contiguous()     # [v | k | q | gate | i | f, W]
+        self.q_col, self.g_col, self.i_col, self.f_col = nv + nk, nv + 2 * nk, 2 * nv + 2 * nk, 2 * nv + 2 * nk + s.heads
+        self.bi, self.bf, self.norm = (self.w(get, p + n, False).reshape(-1) for n in ("i.b", "f.b", "norm"))
+        self.w_o = self.w(get, p + "o", True)
+        if self.bi.numel() != s.heads or self.bf.numel() != s.heads or self.norm.numel() != nv or tuple(self.w_o.shape) != (W, nv):
+            raise ValueError(f"{p}: gate bias / norm / output shapes do not match the mixer's sizes")
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T, dev = b.rows, m.device
+        f32 = dict(dtype=torch.float32, device=dev)
+        u = m.linear(h, self.w_in)                                          # f32 [T, v | k | q | gate | i | f]
+        steps = torch.empty(T, s.heads, 2, **f32)
+        mbuf, mexp = torch.empty(T, s.heads, **f32), torch.empty(T, s.heads, **f32)
+        _call("mrs_hyb_exp_gates", u, u.stride(0), self.i_col, self.f_col, self.q_col, s.heads * s.dim, self.q_mult, self.bi, self.bf, s.gate_cap, self.m_state, steps, mbuf,
+              mexp, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, s.heads)
+        P = s.vdim + 1
+        y = torch.empty(T, s.heads * P, **f32)
+        carry = decay = None
+        if b.segments > b.entries:   # some portion is longer than a segment: scratch for the segments' local end states
+            carry = torch.empty(b.segments, s.heads, s.dim, P, **f32)
+            decay = torch.empty(b.segments, s.heads, **f32)
+        _call("mrs_hyb_gated_scan", u, u.stride(0), steps, self.state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, carry, decay, T, b.entries,
+              b.segments, s.heads, s.vdim, s.dim, s.heads, 1)
+        o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=dev)
+        _call("mrs_hyb_head_norm_gate", y, P, mexp, self.norm, 1, u[:, self.g_col:], u.stride(0), 1, o, T, s.heads, s.vdim, m.spec.eps, m.dt)
+        m.linear(o, self.w_o, out=x, accumulate=accumulate)
+
+
+class ParallelMixer(_Module):
+    """Two registered mixers (tensors under `left.` / `right.`) read the same input; result = (left / rms(left) * w_left + right / rms(right) * w_right) / 2, the norms over
+    the model width with plain weights `left.out` / `right.out`.  Pages, taps and states are the sub-mixers' own."""
+
+    def __init__(self, model, spec: ParallelSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+        self.left = MIXERS[spec.left_kind](model, spec.left, prefix + "left.")
+        self.right = MIXERS[spec.right_kind](model, spec.right, prefix + "right.")
+
+    def carried(self):
+        return tuple(self.left.carried()) + tuple(self.right.carried())
+
+    def kv_bytes_per_token(self) -> int:
+        return sum(c.kv_bytes_per_token() for c in (self.left, self.right) if hasattr(c, "kv_bytes_per_token"))
+
+    def state_bytes_per_slot(self) -> int:
+        return sum(c.state_bytes_per_slot() for c in (self.left, self.right) if hasattr(c, "state_bytes_per_slot"))
+
+    def load(self, get):
+        self.left.load(get)
+        self.right.load(get)
+        self.w_left, self.w_right = self.w(get, self.p + "left.out", False), self.w(get, self.p + "right.out", False)
+        if self.w_left.numel() != self.m.spec.width or self.w_right.numel() != self.m.spec.width:
+            raise ValueError(f"{self.p}: the output norms run over the model width")
+
+    def share_from(self, other: "ParallelMixer") -> None:
+        self.left.share_from(other.left)
+        self.right.share_from(other.right)
+        self.w_left, self.w_right = other.w_left, other.w_right
+
+    def forward(self, h, x, b: RaggedBatch, accumulate: bool = True):
+        m = self.m
+        yl = torch.empty(b.rows, m.spec.width, dtype=torch.float32, device=m.device)
+        yr = torch.empty_like(yl)
+        self.left.forward(h, yl, b, accumulate=False)
+        self.right.forward(h, yr, b, accumulate=False)
+        _call("mrs_hyb_norm_pair_add", x, x.stride(0), yl, self.w_left, yr, self.w_right, b.rows, m.spec.width, m.spec.eps, 0.5, int(accumulate))
+
+
+class TopkSoftmaxReluSqMoe(_Module):
+    """Router logits (weight and bias) in f32; the `top` largest are chosen, their weights are the softmax over the chosen logits only, applied to the experts' OUTPUTS.
+    Expert (no biases, no gate): down(max(up h, 0)^2).  All experts of a step run as grouped products over expert-sorted rows."""
+    wants_f32_input = True
+
+    def __init__(self, model, spec: TopkSoftmaxMoeSpec, prefix: str):
+        super().__init__(model)
+        self.s, self.p = spec, prefix
+
+    def load(self, get):
+        s, p, m = self.s, self.p, self.m
+        dev, dt = m.device, m.torch_dtype
+        self.w_up = torch.stack([get(f"{p}e{e}.up") for e in range(s.experts)]).to(dev, dt).contiguous()       # [E, ff, W]
+        self.w_down = torch.stack([get(f"{p}e{e}.down") for e in range(s.experts)]).to(dev, dt).contiguous()   # [E, W, ff]
+        self.w_router, self.b_router = self.w(get, p + "router", False), self.w(get, p + "router.b", False).reshape(-1)
+        if tuple(self.w_up.shape[1:]) != (s.ff, m.spec.width) or tuple(self.w_down.shape[1:]) != (m.spec.width, s.ff) or \
+                tuple(self.w_router.shape) != (s.experts, m.spec.width) or self.b_router.numel() != s.experts:
+            raise ValueError(f"{p}: expert / router shapes do not match the layer's sizes")
+
+    def forward(self, h, h32, x, b: RaggedBatch, accumulate: bool = True):
+        s, m = self.s, self.m
+        T, W, dev = b.rows, m.spec.width, m.device
+        R = T * s.top
+        ids = torch.empty(R, dtype=torch.int32, device=dev)
+        wts = torch.empty(R, dtype=torch.float32, device=dev)
+        _call("mrs_hyb_route_topk_softmax", h32, self.w_router, self.b_router, T, W, s.experts, s.top, 1.0, ids, wts)
+        meta = torch.empty(s.experts + 1 + 3 * R, dtype=torch.int32, device=dev)
+        bounds, sorted_route, route_pos, sorted_expert = meta[:s.experts + 1], meta[s.experts + 1:][:R], meta[s.experts + 1 + R:][:R], meta[s.experts + 1 + 2 * R:][:R]
+        _call("mrs_hyb_moe_dispatch", ids, R, s.experts, bounds, sorted_route, route_pos, sorted_expert)
+        f32 = dict(dtype=torch.float32, device=dev)
+        if R <= m.GROUPED_GEMV_ROWS:
+            # decode-sized steps: every route streams its expert's slabs; the row gather and the squared ReLU happen in the consuming product's operand load (same roundings)
+            up = torch.empty(R, s.ff, **f32)
+            m.gemv_act(h32, self.w_up, up, R, s.ff, W, h32.stride(0), W, sorted_expert, self.w_up.stride(0), 2, sorted_route, s.top)
+            d = torch.empty(R, W, **f32)
+            m.gemv_act(up, self.w_down, d, R, W, s.ff, s.ff, s.ff, sorted_expert, self.w_down.stride(0), 5)
+        else:
+            xs = torch.empty(R, W, dtype=m.torch_dtype, device=dev)
+            _call("mrs_hyb_moe_gather", h32, sorted_route, None, s.top, xs, R, W, m.dt)
+            up = m.grouped_linear(xs, self.w_up, bounds, sorted_expert)
+            act = torch.empty(R, s.ff, dtype=m.torch_dtype, device=dev)
+            _call("mrs_hyb_relu_sq", up, act, R, s.ff, m.dt)
+            d = m.grouped_linear(act, self.w_down, bounds, sorted_expert)
+        _call("mrs_hyb_moe_combine_weighted", x, d, route_pos, wts, s.top, None, T, W, int(accumulate))
+
+
+MIXERS: Dict[str, Callable] = {"delta_rule": DeltaRuleMixer, "mlstm": MlstmMixer, "parallel": ParallelMixer, "mamba2": Mamba2Mixer, "attention": WindowAttention, "talk_attention": TalkSigmoidAttention, "sink_attention": GatedSinkAttention,
                                "retention": RetentionMixer, "latent_attention": LatentAttention}
-FEED_FORWARDS: Dict[str, Callable] = {"moe": SigmoidMoe, "moe_softmax_clamped": ClampedSoftmaxMoe, "dense_xielu": XieluFeedForward, "dense_glu_silu": GluFeedForward}
+FEED_FORWARDS: Dict[str, Callable] = {"moe_topk_softmax_relu2": TopkSoftmaxReluSqMoe, "moe": SigmoidMoe, "moe_softmax_clamped": ClampedSoftmaxMoe, "dense_xielu": XieluFeedForward, "dense_glu_silu": GluFeedForward}
 
 
 class _Layer:
@@ -1033,7 +1388,7 @@ class HybridDecoder:
         sp = self.spec
         f32 = lambda n: get(n).to(self.device, torch.float32).contiguous()
         self.embed = get(sp.embed).to(self.device, self.torch_dtype).contiguous()
-        self.head = get(sp.head).to(self.device, self.torch_dtype).contiguous()
+        self.head = self.embed if sp.head == sp.embed else get(sp.head).to(self.device, self.torch_dtype).contiguous()   # a head tied to the embedding is the same tensor
         norm = lambda n: (f32(n), f32(n + ".b") if sp.norm == "layer" else None)
         self.final_norm = norm(sp.final_norm)
         if tuple(self.embed.shape) != (sp.vocab, sp.width) or tuple(self.head.shape) != (sp.vocab, sp.width):
@@ -1052,6 +1407,8 @@ class HybridDecoder:
             return w_in, (w_out * np.float32(sp.residual_mult)).contiguous(), mix
         self.multi_stream = bool(sp.streams) or sp.residual_mult != 1.0
         for l in self.layers:
+            if l.spec.weights_of is not None:
+                continue
             if self.multi_stream:
                 l.hc1 = hyper(l.spec.prefix + "hc1")
                 l.hc2 = hyper(l.spec.prefix + "hc2") if l.ff else None
@@ -1062,6 +1419,11 @@ class HybridDecoder:
                 l.norm2 = norm(l.spec.prefix + "norm2")
                 l.norm2b = norm(l.spec.prefix + "norm2b") if sp.post_norms else None
                 l.ff.load(get)
+        for l in self.layers:   # layers that use another layer's tensors: the same norms and feed-forward, the same mixer weights around pages / taps / states of their own
+            if l.spec.weights_of is not None:
+                o = self.layers[l.spec.weights_of]
+                l.norm1, l.norm2, l.norm1b, l.norm2b, l.hc1, l.hc2, l.ff = o.norm1, o.norm2, o.norm1b, o.norm2b, o.hc1, o.hc2, o.ff
+                l.mixer.share_from(o.mixer)
 
     @classmethod
     def from_pretrained(cls, path: str, device, dtype: str = "bfloat16", **kw) -> "HybridDecoder":
@@ -1138,7 +1500,24 @@ class HybridDecoder:
         """The norm in front of a sublayer (and of the head), of the kind the model's description names."""
         if self.spec.norm == "layer":
             return self.layer_norm(x, wb, want32)
-        return self.norm(x, wb[0], one_plus=True, want32=want32)
+        return self.norm(x, wb[0], one_plus=self.spec.norm == "rms_one_plus", want32=want32)
+
+    def pre_norm_pair(self, x, wb1, wb2, want32: bool = False):
+        """The norms in front of two sublayers that read the same rows: one pass, one root mean square, two weights.  Returns (first, second, second in f32 | None)."""
+        if self.spec.norm == "layer":
+            return (self.layer_norm(x, wb1),) + tuple(self.layer_norm(x, wb2, True) if want32 else (self.layer_norm(x, wb2), None))
+        rows, width = x.shape
+        o1 = torch.empty(rows, width, dtype=self.torch_dtype, device=self.device)
+        o2 = torch.empty_like(o1)
+        o32 = torch.empty(rows, width, dtype=torch.float32, device=self.device) if want32 else None
+        _call("mrs_hyb_rmsnorm_pair", x, x.stride(0), wb1[0], wb2[0], o1, o2, o32, rows, width, self.spec.eps, int(self.spec.norm == "rms_one_plus"), self.dt)
+        return o1, o2, o32
+
+    def round_cols(self, u, n: int):
+        """The first n columns of the f32 rows u, rounded once to the serving dtype and contiguous: a column block of one product as the operand of the next."""
+        out = torch.empty(u.shape[0], n, dtype=self.torch_dtype, device=self.device)
+        _call("mrs_hyb_round_cols", u, u.stride(0), out, u.shape[0], n, self.dt)
+        return out
 
     def add_post_norm(self, x, y, in_bias, wb, then=None, want32: bool = False):
         """x += norm(y + in_bias): a sublayer's product (its bias still to be added) joins the f32 residual stream through the norm behind the sublayer.  `then` = the
@@ -1222,6 +1601,10 @@ class HybridDecoder:
                     h_next = self.add_post_norm(x, y, l.ff.out_bias, l.norm2b, then=nxt)
                 else:
                     h_next = self.add_post_norm(x, y, l.mixer.out_bias, l.norm1b, then=nxt)
+            elif sp.parallel_sublayers and l.ff:
+                h1, h2, h32 = self.pre_norm_pair(x, l.norm1, l.norm2, want32=l.ff.wants_f32_input)   # both sublayers read the row as it is now; their sums join it in turn
+                l.mixer.forward(h1, x, b)
+                l.ff.forward(h2, h32, x, b)
             else:
                 l.mixer.forward(self.pre_norm(x, l.norm1), x, b)
                 if l.ff:
@@ -1436,7 +1819,7 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
     return get
 
 
-SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec, "Sobunex": sobunex_spec, "Setopel": setopel_spec}
+SPEC_READERS: Dict[str, Callable[[dict], HybridSpec]] = {"Gekilix": gekilix_spec, "Sobunex": sobunex_spec, "Setopel": setopel_spec, "Gifopel": gifopel_spec}
 
 
 class HybridCache:

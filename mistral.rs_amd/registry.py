@@ -34,6 +34,12 @@ def _load_setopel(path: str, device, dtype: str = "bfloat16", **kw):
     return HybridDecoder.from_pretrained(path, device, dtype, **kw)
 
 
+@register("Gifopel")
+def _load_gifopel(path: str, device, dtype: str = "bfloat16", **kw):
+    from .hybrid import HybridDecoder
+    return HybridDecoder.from_pretrained(path, device, dtype, **kw)
+
+
 @register("llama")
 def _load_llama_gguf(path: str, device, dtype: str = "bfloat16", **kw):
     from .gguf.archive import load_llama
