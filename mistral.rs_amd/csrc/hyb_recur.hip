@@ -355,10 +355,13 @@ extern "C" int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, co
   int R = lanes_per_column;
   if (R != 4 && R != 16) R = ((long long)entries * H * ((Dv + 15) / 16) >= 1024 || D < 64) ? 4 : 16;
   const int PT = 64 / R;
-  const int nw_all = (Dv + PT - 1) / PT, nw = nw_all > 8 ? 8 : nw_all, nblk = (nw_all + nw - 1) / nw;
   const int perp = (per + 3) & ~3, rowlen = 2 * D + perp + Dv + 1, rowpad = (rowlen + 3) & ~3;
   constexpr int TC = 4, MAXC = 8;
-  if (rowpad > MAXC * 64 * nw) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers (key size far above value size)");
+  const int nw_all = (Dv + PT - 1) / PT, nw_stage = (rowpad + MAXC * 64 - 1) / (MAXC * 64);  // waves for the columns; waves whose registers can stage a row of operands
+  int nw = nw_all > 8 ? 8 : nw_all;
+  const int nblk = (nw_all + nw - 1) / nw;
+  if (nw < nw_stage) nw = nw_stage;  // few value columns next to long keys: further waves only help to stage (their columns lie past Dv and are never written)
+  if (nw > 8) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers");
   const size_t lds = (size_t)2 * TC * rowpad * 4;
   if (lds > 65536) return fail("mrs_hyb_delta_scan: staged rows above 64 KB");
   const bool vec = D % 4 == 0;

@@ -1735,14 +1735,52 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
     g = torch.Generator(device=device).manual_seed(seed)
     shapes: Dict[str, tuple] = {spec.embed: (spec.vocab, W), spec.head: (spec.vocab, W), spec.final_norm: (W,)}
     norm_names = {spec.final_norm} | ({spec.embed_norm} if spec.embed_norm else set())
+    def new_mixer_shapes(p, m) -> bool:
+        """delta-rule, matrix-memory, parallel and chunked / gated attention mixers; False: `m` is of another kind"""
+        if isinstance(m, ParallelSpec):
+            shapes.update({p + "left.out": (W,), p + "right.out": (W,)})
+            norm_like.update({p + "left.out", p + "right.out"})
+            for side, sub in (("left.", m.left), ("right.", m.right)):
+                if not new_mixer_shapes(p + side, sub):
+                    raise ValueError("synthetic_weights: a parallel mixer's sides are attention, delta-rule or matrix-memory mixers")
+        elif isinstance(m, DeltaRuleSpec):
+            nqk, nv, rank = m.kv_heads * m.dim, m.heads * m.vdim, max(8, min(128, W // 16))
+            for n, rows in (("q", nqk), ("k", nqk), ("v", nv)):
+                shapes.update({p + n: (rows, W), p + n + ".conv": (rows, m.conv)})
+            shapes.update({p + "b": (m.heads, W), p + "A_log": (m.heads,), p + "norm": (m.vdim,), p + "o": (W, nv)})
+            if m.decay == "channel":
+                shapes.update({p + "a1": (rank, W), p + "a2": (m.heads * m.dim, rank), p + "dt_bias": (m.heads * m.dim,)})
+            else:
+                shapes.update({p + "a": (m.heads, W), p + "dt_bias": (m.heads,)})
+            shapes.update({p + "g1": (rank, W), p + "g2": (nv, rank)} if m.gate == "sigmoid_lowrank" else {p + "g": (nv, W)})
+        elif isinstance(m, MlstmSpec):
+            nk, nv = m.heads * m.dim, m.heads * m.vdim
+            shapes.update({p + "q": (nk, W), p + "k": (nk, W), p + "v": (nv, W), p + "g": (nv, W), p + "o": (W, nv), p + "norm": (nv,), p + "i": (m.heads, W), p + "i.b": (m.heads,),
+                           p + "f": (m.heads, W), p + "f.b": (m.heads,)})
+        elif isinstance(m, AttentionSpec) and (m.head_norm or m.sink or m.head_gate):
+            shapes.update({p + "q": (m.heads * m.dim, W), p + "k": (m.kv_heads * m.dim, W), p + "v": (m.kv_heads * m.vdim, W), p + "o": (W, m.heads * m.vdim),
+                           p + "q.norm": (m.dim if m.head_norm else m.heads * m.dim,), p + "k.norm": (m.dim if m.head_norm else m.kv_heads * m.dim,)})
+            if m.sink:
+                shapes[p + "sink"] = (m.heads,)
+            if m.head_gate:
+                shapes[p + "g"] = (m.heads, W)
+        else:
+            return False
+        return True
+
+    norm_like = set()   # plain-weight norms besides the layers' own: drawn around one
     for ls in spec.layers:
         p, m = ls.prefix, ls.mixer
+        if ls.weights_of is not None:
+            continue
         for n in ["norm1"] + (["norm2"] if ls.ff else []) + ((["norm1b"] + (["norm2b"] if ls.ff else [])) if spec.post_norms else []):
             norm_names.add(p + n)
         if spec.streams:
             for q in ("hc1", "hc2") if ls.ff else ("hc1",):
                 shapes.update({f"{p}{q}.in": (spec.streams,), f"{p}{q}.out": (spec.streams,), f"{p}{q}.mix": (spec.streams, spec.streams)})
-        if isinstance(m, SinkAttentionSpec):
+        if new_mixer_shapes(p + "mix.", m):
+            pass
+        elif isinstance(m, SinkAttentionSpec):
             own = ["q", "k", "v"] if m.kv_from is None else ["q"]
             rows = {"q": m.heads * m.dim, "k": m.kv_heads * m.dim, "v": m.kv_heads * m.vdim}
             for n in own:
@@ -1771,6 +1809,10 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
             shapes.update({p + "mlp.gate": (ls.ff.ff, W), p + "mlp.up": (ls.ff.ff, W), p + "mlp.down": (W, ls.ff.ff)})
         elif isinstance(ls.ff, DenseSpec):
             shapes.update({p + "mlp.up": (ls.ff.ff, W), p + "mlp.up.b": (ls.ff.ff,), p + "mlp.down": (W, ls.ff.ff), p + "mlp.down.b": (W,), p + "mlp.act": (2,)})
+        elif isinstance(ls.ff, TopkSoftmaxMoeSpec):
+            shapes.update({p + "mlp.router": (ls.ff.experts, W), p + "mlp.router.b": (ls.ff.experts,)})
+            for e in range(ls.ff.experts):
+                shapes.update({f"{p}mlp.e{e}.up": (ls.ff.ff, W), f"{p}mlp.e{e}.down": (W, ls.ff.ff)})
         elif ls.ff:
             f = ls.ff
             shapes[p + "mlp.router"] = (f.experts, W)
@@ -1789,8 +1831,11 @@ def synthetic_weights(spec: HybridSpec, device, seed: int = 0) -> Callable[[str]
         shape = shapes[name]
         r = torch.randn(*shape, device=device, generator=g)
         last = name.rsplit(".", 1)[-1]
-        if name.endswith(("q.norm", "k.norm", "dkv.norm")) or last == "D" or name.endswith("mix.norm") or (name in norm_names and spec.norm == "layer"):
+        if name.endswith(("q.norm", "k.norm", "dkv.norm")) or last == "D" or name.endswith(("mix.norm", "left.norm", "right.norm")) or name in norm_like or \
+                (name in norm_names and spec.norm in ("layer", "rms")):
             r = 1.0 + 0.1 * r
+        elif name.endswith("f.b"):
+            r = 3.0 + 0.5 * r      # forget gates mostly open
         elif last == "mix" and len(shape) == 2 and shape[0] == shape[1] == spec.streams:
             r = torch.eye(shape[0], device=device) + 0.1 * r
         elif last == "in" and shape == (spec.streams,):
