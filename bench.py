@@ -1054,6 +1054,240 @@ def setopel_leg(a, dev):
                       "config": {"model": f"setopel-{a.setopel}", "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "setopel": out}), flush=True)
 
 
+GIFOPEL_SIZES = {
+    # layer lists that resemble a small, a mid-size and a large decoder: matrix memory, chunked attention beside a delta rule, and a delta rule with channel decays in turn
+    "s": dict(width=1024, layers=6, heads=16, kv=4, dim=64, vdim=64, chunk=1024, d_heads=8, d_kv=8, d_dim=64, d_vdim=128, r_heads=8, r_kv=4, r_dim=64, r_vdim=64, m_heads=8, m_dim=64,
+              m_vdim=128, conv=4, ff=2816, experts=32, top=4, eff=512, vocab=32000),
+    "m": dict(width=2048, layers=6, heads=16, kv=4, dim=128, vdim=128, chunk=2048, d_heads=16, d_kv=16, d_dim=128, d_vdim=128, r_heads=8, r_kv=4, r_dim=128, r_vdim=128, m_heads=8,
+              m_dim=128, m_vdim=256, conv=4, ff=5632, experts=64, top=6, eff=768, vocab=32000),
+    "l": dict(width=4096, layers=3, heads=32, kv=8, dim=128, vdim=128, chunk=4096, d_heads=32, d_kv=32, d_dim=128, d_vdim=128, r_heads=16, r_kv=8, r_dim=128, r_vdim=128, m_heads=16,
+              m_dim=128, m_vdim=256, conv=4, ff=11008, experts=64, top=6, eff=1408, vocab=32000),
+}
+
+
+def gifopel_leg(a, dev):
+    """`--gifopel SIZE`: prefill and decode throughput of a Gifopel layer list (paired norms; matrix memory, chunked sink attention beside a delta rule, delta rule with channel
+    decays; dense and routed squared-ReLU feed-forwards; bf16 weights, random) beside the closest model of the package at equal size: state-space layers of equal state size
+    in place of the recurrent mixers, windowed softmax attention (window = the chunk) in place of the chunked one, sigmoid-routed GLU experts of equal weight bytes.  Then the
+    kernels of the two designs that do like work, one launch each at the model's shapes: time and the fraction of the roofline (8 TB/s for what a kernel must read and
+    write; prompt attention and the recurrences run on the f32 vector ALU in both designs and are priced in FLOP/s of the work done)."""
+    import torch
+    from mistralrs_amd.hybrid import (AttentionSpec, DeltaRuleSpec, GluSpec, HybridCache, HybridDecoder, HybridSpec, LayerSpec, Mamba2Spec, MlstmSpec, MoeSpec, ParallelSpec,
+                                      RaggedBatch, RotarySpec, TopkSoftmaxMoeSpec, _call, synthetic_weights)
+    z = GIFOPEL_SIZES[a.gifopel]
+    W, H, G, D, Dv = z["width"], z["heads"], z["kv"], z["dim"], z["vdim"]
+    new_layers, old_layers = [], []
+    for i in range(z["layers"]):
+        kind = ("mlstm", "parallel", "channel_delta")[i % 3]
+        ff_new = GluSpec(z["ff"]) if i == 0 else TopkSoftmaxMoeSpec(z["experts"], z["top"], z["eff"])
+        ff_old = GluSpec(z["ff"]) if i == 0 else MoeSpec(z["experts"], z["top"], 2 * z["eff"] // 3)
+        if kind == "mlstm":
+            new_layers.append(LayerSpec("mlstm", MlstmSpec(z["m_heads"], z["m_dim"], z["m_vdim"], 15.0), ff_new, f"l{i}."))
+            old_layers.append(LayerSpec("mamba2", Mamba2Spec(z["m_heads"], z["m_vdim"], z["m_dim"], z["m_heads"], z["conv"], 1), ff_old, f"l{i}."))
+        elif kind == "parallel":
+            left = AttentionSpec(H, G, D, Dv, D ** -0.5, 0, 0, RotarySpec(D // 2, 500000.0), True, chunk=z["chunk"], head_norm=True, sink=True, head_gate=True)
+            right = DeltaRuleSpec(z["r_heads"], z["r_kv"], z["r_dim"], z["r_vdim"], z["conv"], "head", "silu")
+            new_layers.append(LayerSpec("parallel", ParallelSpec("attention", left, "delta_rule", right), ff_new, f"l{i}."))
+            old_layers.append(LayerSpec("attention", AttentionSpec(H, G, D, Dv, D ** -0.5, z["chunk"], 0, RotarySpec(D // 2, 500000.0)), None, f"l{i}a."))
+            old_layers.append(LayerSpec("mamba2", Mamba2Spec(z["r_heads"], z["r_vdim"], z["r_dim"], z["r_kv"], z["conv"], 1), ff_old, f"l{i}."))
+        else:
+            new_layers.append(LayerSpec("delta_rule", DeltaRuleSpec(z["d_heads"], z["d_kv"], z["d_dim"], z["d_vdim"], z["conv"], "channel", "sigmoid_lowrank"), ff_new, f"l{i}."))
+            old_layers.append(LayerSpec("mamba2", Mamba2Spec(z["d_heads"], z["d_vdim"], z["d_dim"], z["d_kv"], z["conv"], 1), ff_old, f"l{i}."))
+    specs = {"gifopel": HybridSpec(z["vocab"], W, 1e-6, new_layers, head="embed", norm="rms", parallel_sublayers=True),
+             "state_space_window_attention_moe": HybridSpec(z["vocab"], W, 1e-6, old_layers)}
+    prompts, batches, bs, ctx = [512, 2048], [1, 8], 32, 512
+    max_tok = max(prompts) + a.warmup + a.steps + 64
+
+    def timed(fn, reps):
+        fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / reps
+
+    out = {"sizes": z, "dtype": "bf16", "weights": "random, drawn on the device", "models": {}, "kernels": {}}
+    keep = {}
+    with torch.no_grad():
+        for name, spec in specs.items():
+            model = HybridDecoder(spec, dev, "bfloat16", num_blocks=max(batches) * (-(-max_tok // bs) + 1) + 2, block_size=bs, state_slots=max(batches))
+            model.load_weights(synthetic_weights(spec, dev, 0))
+            cache = HybridCache(model)
+            r = {"prefill": {}, "decode": {}}
+            for T in prompts:
+                assert cache.reserve(1, T)
+                b = RaggedBatch.build([cache.entry(1, [(1000 + i) % z["vocab"] for i in range(T)], 0, [T - 1])], bs, dev)
+                t = timed(lambda: model.forward_batch(b), 3)
+                r["prefill"][str(T)] = {"tokens_per_sec": round(T / t, 1), "ms": round(1e3 * t, 3)}
+                cache.release(1)
+            for nb in batches:
+                for q in range(nb):
+                    assert cache.reserve(q + 1, ctx + a.warmup + a.steps + 2)
+                model.forward_batch(RaggedBatch.build([cache.entry(q + 1, [(1000 + i + q) % z["vocab"] for i in range(ctx)], 0, []) for q in range(nb)], bs, dev))
+                g = model.capture_decode(nb, -(-(ctx + a.warmup + a.steps + 2) // bs))
+                pos = ctx
+
+                def step():
+                    nonlocal pos
+                    g.replay([cache.entry(q + 1, [7 + q], pos) for q in range(nb)])
+                    pos += 1
+                for _ in range(a.warmup):
+                    step()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(a.steps):
+                    step()
+                torch.cuda.synchronize()
+                t = (time.perf_counter() - t0) / a.steps
+                r["decode"][f"batch{nb}"] = {"tokens_per_sec": round(nb / t, 1), "ms_per_step": round(1e3 * t, 4)}
+                del g
+                for q in range(nb):
+                    cache.release(q + 1)
+            out["models"][name] = r
+            keep[name] = model
+            torch.cuda.empty_cache()
+        # ---- like kernels of the two designs, one launch each
+        new, old = keep["gifopel"], keep["state_space_window_attention_moe"]
+        kern = out["kernels"]
+        e = 2
+        f32 = dict(dtype=torch.float32, device=dev)
+
+        def pair(label, t_new, t_old, nbytes=None, flops=None, **extra):
+            d = {"gifopel_us": round(1e6 * t_new, 1), "other_us": round(1e6 * t_old, 1), "time_ratio": round(t_new / t_old, 2), **extra}
+            if nbytes is not None:
+                d.update(min_bytes=nbytes[0], other_min_bytes=nbytes[1], gifopel_hbm_frac=round(nbytes[0] / t_new / HBM_PEAK, 4), other_hbm_frac=round(nbytes[1] / t_old / HBM_PEAK, 4))
+            if flops is not None:
+                d.update(flops=flops[0], other_flops=flops[1], gifopel_tflops=round(flops[0] / t_new / 1e12, 2), other_tflops=round(flops[1] / t_old / 1e12, 2))
+            kern[label] = d
+        mem, both, cdel = new.layers[0].mixer, new.layers[1].mixer, new.layers[2].mixer
+        ossm_m, oattn, ossm_r, ossm_d = old.layers[0].mixer, old.layers[1].mixer, old.layers[2].mixer, old.layers[3].mixer
+
+        def ssd(b, m2):
+            ms = m2.s
+            T = b.rows
+            uo = torch.randn(T, 2 * ms.inner + 2 * ms.groups * ms.state + ms.heads, **f32) * 0.1
+            xbc = torch.randn(T, ms.conv_channels, **f32) * 0.1
+            yy, steps = torch.empty(T, ms.inner, **f32), torch.empty(T, ms.heads, 2, **f32)
+            carry, dk = torch.empty(b.segments, ms.heads, ms.state, ms.vdim, **f32), torch.empty(b.segments, ms.heads, **f32)
+            return lambda: _call("mrs_hyb_ssd_scan", xbc, uo, m2.dt_bias, m2.A_log, m2.D, m2.ssm_state, yy, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0,
+                                 steps, carry, dk, T, b.entries, b.segments, ms.conv_channels, uo.stride(0), ms.inner + ms.conv_channels, ms.heads, ms.vdim, ms.state, ms.groups)
+        for label, ents in (("prompt_2048", [(0, 2048, 0)]), ("prompt_8x256", [(0, 256, q) for q in range(8)]), ("decode_batch8", [(600, 1, q) for q in range(8)]),
+                            ("decode_batch1", [(600, 1, 0)])):
+            b = RaggedBatch.build([{"tokens": [0] * n, "pos0": p0, "slot": sl, "blocks": list(range(1, 2 + (p0 + n) // bs)), "want": []} for p0, n, sl in ents], bs, dev)
+            T = b.rows
+            portion = T > b.entries
+            # delta rule, a decay per key channel / per head
+            for tag, mx, o2 in (("channel", cdel, ossm_d), ("head", both.right, ossm_r)):
+                sp = mx.s
+                c = torch.randn(T, mx.channels, **f32) * 0.1
+                beta, dec, yy = torch.rand(T, sp.heads, **f32), 1 - 0.1 * torch.rand(T, sp.heads * mx.per, **f32), torch.empty(T, mx.nv, **f32)
+                t_new = timed(lambda: _call("mrs_hyb_delta_scan", c, mx.channels, beta, dec, mx.state, yy, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, sp.heads, sp.kv_heads,
+                                            sp.dim, sp.vdim, mx.per, 0), 5)
+                t_old = timed(ssd(b, o2), 5)
+                st = sp.heads * sp.dim * sp.vdim
+                nbytes = T * 4 * (mx.channels + mx.nv + sp.heads * (1 + mx.per)) + len(ents) * 8 * st
+                pair(f"delta_{tag}_decay_{label}", t_new, t_old, (nbytes, T * 4 * (o2.s.conv_channels + o2.s.inner) + len(ents) * 8 * st),
+                     (7.0 * T * st, 4.0 * T * st * (3 if portion and b.segments > b.entries else 1)))
+            # matrix memory: gates + scan with the normaliser column + normaliser / head norm / gate
+            sp = mem.s
+            nv, nk = sp.heads * sp.vdim, sp.heads * sp.dim
+            u = torch.randn(T, 2 * nv + 2 * nk + 2 * sp.heads, **f32) * 0.1
+            steps, mbuf, mexp = torch.empty(T, sp.heads, 2, **f32), torch.empty(T + b.entries, sp.heads, **f32), torch.empty(T, sp.heads, **f32)
+            yy = torch.empty(T, sp.heads * (sp.vdim + 1), **f32)
+            carry, dk = torch.empty(b.segments, sp.heads, sp.dim, sp.vdim + 1, **f32), torch.empty(b.segments, sp.heads, **f32)
+            t_g = timed(lambda: _call("mrs_hyb_exp_gates", u, u.stride(0), mem.i_col, mem.f_col, mem.bi, mem.bf, 15.0, mem.m_state, steps, mbuf, mexp, b.tok_seq, b.seq_start,
+                                      b.seq_pos0, b.seq_slot, T, b.entries, sp.heads), 5)
+            t_s = timed(lambda: _call("mrs_hyb_gated_scan", u, u.stride(0), steps, mem.state, yy, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, carry, dk, T,
+                                      b.entries, b.segments, sp.heads, sp.vdim, sp.dim, sp.heads, 1, mem.q_mult), 5)
+            t_old = timed(ssd(b, ossm_m), 5)
+            st = sp.heads * sp.dim * sp.vdim
+            fl = 4.0 * T * st * (3 if b.segments > b.entries else 1)
+            pair(f"matrix_memory_gates_and_scan_{label}", t_g + t_s, t_old, None, (fl, fl), gates_us=round(1e6 * t_g, 1), scan_us=round(1e6 * t_s, 1))
+        # attention: 2048-token prompt inside one chunk / window, decode
+        bps = -(-(2048 + 64) // bs)
+        att = both.left
+        for c_ in (att.k_cache, att.v_cache, oattn.k_cache, oattn.v_cache):
+            c_.normal_()
+        for label, nseq, p0, n in (("attention_prompt_2048", 1, 0, 2048), ("attention_decode_batch8_ctx2048", 8, 2047, 1), ("attention_decode_batch1_ctx2048", 1, 2047, 1)):
+            ents = [{"tokens": [0] * n, "pos0": p0, "slot": 0, "blocks": list(range(1 + q * bps, 1 + (q + 1) * bps)), "want": []} for q in range(nseq)]
+            if ents[-1]["blocks"][-1] >= new.num_blocks:
+                continue
+            b = RaggedBatch.build(ents, bs, dev)
+            T = b.rows
+            qn = torch.randn(T, H * D, device=dev).to(torch.bfloat16)
+            gate = torch.randn(T, H, **f32)
+            o = torch.empty(T, H * Dv, dtype=torch.bfloat16, device=dev)
+            seg = (b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT)
+            ch = max(z["chunk"], 2048)
+            t_new = timed(lambda: _call("mrs_hyb_paged_attn_chunked", qn, att.k_cache, att.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, ch,
+                                        D ** -0.5, 1, *seg, 0.0, 1, att.sink, gate, H, 1, *new.key_splits(b, H, Dv, ch)), 5)
+            t_old = timed(lambda: _call("mrs_hyb_paged_window_attn", qn, oattn.k_cache, oattn.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, H, G, D, Dv, bs, b.max_blocks, ch, 0,
+                                        D ** -0.5, 1, *seg), 5)
+            pairs = sum(p0 + i + 1 for i in range(n)) * nseq
+            fl = 2.0 * pairs * H * (D + Dv)
+            kvb = nseq * e * G * (D + Dv) * (p0 + n) + T * e * H * (D + Dv)
+            pair("chunked_sink_" + label, t_new, t_old, (kvb, kvb), (fl, fl))
+        # row-wise kernels at 2048 rows
+        T = 2048
+        b = RaggedBatch.build([{"tokens": [0] * T, "pos0": 0, "slot": 0, "blocks": list(range(1, 2 + T // bs)), "want": []}], bs, dev)
+        x, wv, wv2 = torch.randn(T, W, **f32), torch.randn(W, **f32), torch.randn(W, **f32)
+        ob, ob2, o32 = torch.empty(T, W, dtype=torch.bfloat16, device=dev), torch.empty(T, W, dtype=torch.bfloat16, device=dev), torch.empty(T, W, **f32)
+        t_new = timed(lambda: _call("mrs_hyb_rmsnorm_pair", x, W, wv, wv2, ob, ob2, o32, T, W, 1e-6, 0, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_rmsnorm", x, W, wv, ob, o32, None, T, W, 1, 1e-6, 1, 1, None, 0, 0), 10)
+        pair("two_norms_one_launch_vs_one_norm_2048_rows", t_new, t_old, (T * W * (4 + 2 + 2 + 4), T * W * (4 + 2 + 4)))
+        y1, y2 = torch.randn(T, W, **f32), torch.randn(T, W, **f32)
+        t_new = timed(lambda: _call("mrs_hyb_norm_pair_add", x, W, y1, wv, y2, wv2, T, W, 1e-6, 0.5, 1), 10)
+        pair("normed_average_into_stream_vs_one_norm_2048_rows", t_new, t_old, (T * W * 16, T * W * (4 + 2 + 4)))
+        E, top = z["experts"], z["top"]
+        ids, wts, gt = torch.empty(T * top, dtype=torch.int32, device=dev), torch.empty(T * top, **f32), torch.empty(T, **f32)
+        wr, br = torch.randn(E + 1, W, **f32), torch.randn(E, **f32)
+        t_new = timed(lambda: _call("mrs_hyb_route_topk_softmax", x, wr, br, T, W, E, top, 1.0, ids, wts), 10)
+        t_old = timed(lambda: _call("mrs_hyb_route_sigmoid_topk", x, wr, T, W, E, top, 0, ids, wts, gt), 10)
+        pair("router_2048_rows", t_new, t_old, (T * W * 4 + E * W * 4, T * W * 4 + E * W * 4))
+        ff = z["eff"]
+        R_ = T * top
+        up, gu = torch.randn(R_, ff, **f32), torch.randn(R_, 2 * ff, **f32)
+        act = torch.empty(R_, ff, dtype=torch.bfloat16, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_relu_sq", up, act, R_, ff, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_glu_silu", gu, act, R_, ff, 1), 10)
+        pair("expert_activation_prompt", t_new, t_old, (R_ * ff * 6, R_ * ff * 10))
+        sp = cdel.s
+        yv, gv, nw_ = torch.randn(T, cdel.nv, **f32), torch.randn(T, cdel.nv, **f32), torch.randn(cdel.nv, **f32)
+        ov = torch.empty(T, cdel.nv, dtype=torch.bfloat16, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_head_norm_gate", yv, sp.vdim, None, nw_, 0, gv, cdel.nv, 1, ov, T, sp.heads, sp.vdim, 1e-6, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_rmsnorm", yv, cdel.nv, nw_, ov, None, None, T, cdel.nv, sp.heads, 1e-6, 0, 1, gv, cdel.nv, 0), 10)
+        pair("head_norm_gate_vs_gated_group_norm_2048_rows", t_new, t_old, (T * cdel.nv * 10, T * cdel.nv * 10))
+        # operands of the recurrence: convolution + unit vectors / write strengths / decays against convolution + step sizes
+        uc = torch.randn(T, cdel.w_in.shape[0], **f32)
+        cc = torch.empty(T, cdel.channels, **f32)
+        av = torch.randn(T, sp.heads * cdel.per, **f32)
+        beta, dec = torch.empty(T, sp.heads, **f32), torch.empty(T, sp.heads * cdel.per, **f32)
+
+        def prep():
+            _call("mrs_hyb_conv", uc, uc.stride(0), None, cdel.conv_w, None, cdel.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, cc, T, 1, cdel.channels, sp.conv, 1)
+            _call("mrs_hyb_delta_prep", cc, cdel.channels, uc, uc.stride(0), cdel.b_col, av, av.stride(0), cdel.A_log, cdel.dt_bias, beta, dec, T, sp.heads, sp.kv_heads, sp.dim, cdel.per)
+        ms = ossm_d.s
+        uo = torch.randn(T, ossm_d.w_in.shape[0], **f32)
+        xbc = torch.empty(T, ms.conv_channels, **f32)
+        t_new = timed(prep, 10)
+        t_old = timed(lambda: _call("mrs_hyb_conv_silu", uo[:, ms.inner:], uo.stride(0), ossm_d.conv_w, ossm_d.conv_b, ossm_d.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot,
+                                    xbc, T, 1, ms.conv_channels, ms.conv), 10)
+        pair("conv_and_delta_operands_vs_conv_2048_rows", t_new, t_old, (T * 4 * (2 * cdel.channels + 2 * 2 * cdel.nqk + 2 * sp.heads * cdel.per), T * 8 * ms.conv_channels), launches=3)
+        nqkv = H * D + G * D + G * Dv
+        uq = torch.randn(T, nqkv + H, **f32)
+        ql = torch.empty(T, H * D, dtype=torch.bfloat16, device=dev)
+        t_new = timed(lambda: _call("mrs_hyb_qk_headnorm_rope_cache", uq, nqkv + H, att.q_norm, att.k_norm, att.freq, b.tok_pos, b.slot_mapping, ql, att.k_cache, att.v_cache, T, H, G,
+                                    D, Dv, D // 2, bs, 1e-6, 1), 10)
+        t_old = timed(lambda: _call("mrs_hyb_qk_norm_rope_cache", uq, nqkv + H, oattn.q_norm, oattn.k_norm, oattn.freq, b.tok_pos, b.slot_mapping, ql, oattn.k_cache, oattn.v_cache, T, H,
+                                    G, D, Dv, D // 2, bs, 1e-6, 1), 10)
+        pair("head_norm_rotary_page_write_vs_whole_norm_rotary_page_write", t_new, t_old, (T * nqkv * 6, T * nqkv * 6))
+    d1 = out["models"]["gifopel"]["decode"]["batch1"]
+    print(json.dumps({"metric": "gifopel_decode_tokens_per_sec", "value": d1["tokens_per_sec"], "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+                      "ms_per_step": d1["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                      "config": {"model": f"gifopel-{a.gifopel}", "global_batch": 1, "seq_len": 512, "parallelism": "tp1"}, "gifopel": out}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -1086,7 +1320,18 @@ def main():
     ap.add_argument("--setopel", choices=sorted(SETOPEL_SIZES), default=None,
                     help="instead of the default workload: a Setopel layer list (residual streams; latent / sink attention, retention; SiLU-GLU feed-forwards; bf16) of the given size "
                          "beside an attention + state-space list of the package at equal size, and the like kernels of the two one by one")
+    ap.add_argument("--gifopel", choices=sorted(GIFOPEL_SIZES), default=None,
+                    help="instead of the default workload: a Gifopel layer list (matrix memory, chunked sink attention beside a delta rule, delta rule with channel decays; dense / routed "
+                         "squared-ReLU feed-forwards; bf16) of the given size beside a state-space + windowed-attention + routed-experts list of the package at equal size, and the like "
+                         "kernels of the two one by one")
     a = ap.parse_args()
+    if a.gifopel:
+        import torch
+        dev = torch.device("cuda", 0)
+        torch.cuda.set_device(dev)
+        if a.steps == 256:
+            a.steps = 128
+        return gifopel_leg(a, dev)
     if a.setopel:
         import torch
         dev = torch.device("cuda", 0)

@@ -41,7 +41,7 @@ int mrs_hyb_qkv_bias_temp_cache(const float *qkv, int ld, const float *qb, const
 int mrs_hyb_rotary_half(float *u, int ld, int q_col, int k_col, int heads, int D, int rot, const float *freq, const int *tok_pos, float k_mult, int rows, void *stream);
 int mrs_hyb_latent_norm_cache(const float *u, int ld, int nq, int R, const float *w, const long long *slot_mapping, void *q_out, void *c_cache, float eps, int rows, int dtype, void *stream);
 int mrs_hyb_hyper_step(float *x, const float *y, const float *mix, const float *outw, const float *inw, const float *norm_w, void *out, float *out32, int rows, int S, int W, float eps, int one_plus, int dtype, void *stream);
-int mrs_hyb_gated_scan(const float *xkq, int ld, float *steps, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *carry, float *decay, int rows, int entries, int segments, int heads, int P, int N, int G, int ones, void *stream);
+int mrs_hyb_gated_scan(const float *xkq, int ld, float *steps, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *carry, float *decay, int rows, int entries, int segments, int heads, int P, int N, int G, int ones, float q_mult, void *stream);
 int mrs_hyb_qk_headnorm_rope_cache(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping, void *q_out, void *k_cache, void *v_cache, int rows, int H, int G, int D, int Dv, int rot, int block_size, float eps, int dtype, void *stream);
 int mrs_hyb_paged_attn_chunked(const void *q, const void *k_cache, const void *v_cache, const int *block_tables, const int *tok_seq, const int *tok_pos, void *out, int rows, int H, int G, int D, int Dv, int block_size, int max_blocks, int chunk, float scale, int dtype, const int *seg_entry, const int *seg_row0, const int *seg_len, int segments, int seg_rows, float softcap, int sink, const float *sink_logit, const float *gate, int ldg, int gate_per_head, float *scratch, int splits, void *stream);
 int mrs_hyb_route_topk_softmax(const float *h, const float *wr, const float *bias, int rows, int W, int E, int top, float scale, int *ids, float *wts, void *stream);
@@ -50,7 +50,7 @@ const char *mrs_hyb_recur_last_error();
 int mrs_hyb_rmsnorm_pair(const float *x, int ldx, const float *w1, const float *w2, void *out1, void *out2, float *out2_32, int rows, int W, float eps, int one_plus, int dtype, void *stream);
 int mrs_hyb_delta_prep(float *c, int ldc, const float *u, int ldu, int b_col, const float *a, int lda, const float *A_log, const float *dt_bias, float *beta, float *dec, int rows, int H, int G, int D, int per, void *stream);
 int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, const float *dec, float *state, float *out, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, int G, int D, int Dv, int per, int lanes_per_column, void *stream);
-int mrs_hyb_exp_gates(float *u, int ldu, int i_col, int f_col, int q_col, int nq, float q_mult, const float *bi, const float *bf, float cap, float *m_state, float *steps, float *mbuf, float *mexp, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, void *stream);
+int mrs_hyb_exp_gates(const float *u, int ldu, int i_col, int f_col, const float *bi, const float *bf, float cap, float *m_state, float *steps, float *mbuf, float *mexp, const int *tok_seq, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, void *stream);
 int mrs_hyb_head_norm_gate(const float *y, int ldp, const float *mexp, const float *w, int w_full, const float *gate, int ldg, int gate_mode, void *out, int rows, int H, int Dv, float eps, int dtype, void *stream);
 int mrs_hyb_norm_pair_add(float *x, int ldx, const float *y1, const float *w1, const float *y2, const float *w2, int rows, int W, float eps, float c, int accumulate, void *stream);
 int mrs_hyb_round_cols(const float *u, int ldu, void *out, int rows, int n, int dtype, void *stream);

@@ -229,6 +229,7 @@ struct ScanArgs {
   int C, ldu, dt_col, heads, P, N, G, rows;
   int Pin;            // value columns that xbc carries per head; P - Pin (0 or 1) further columns of the state take x = 1 (a running sum of dt B next to the outer products)
   int ext_steps;      // `steps` was filled by the caller (gates of another form): nothing of dt_bias / A_log / fixed_decay is read
+  float c_mult;       // every C value is multiplied by this when it is read (a query scale)
 };
 __global__ void __launch_bounds__(256) ssd_steps_kernel(ScanArgs a) {
   const int i = blockIdx.x * 256 + threadIdx.x;
@@ -295,7 +296,7 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
         const float4 b4 = *(const float4 *)(xr + (nk ? bcol : inner) + kk), c4 = *(const float4 *)(xr + (nk ? ccol : inner) + kk);
         const bool on = k < nk;
         B_[k] = on ? b4.x : 0.f; B_[k + 1] = on ? b4.y : 0.f; B_[k + 2] = on ? b4.z : 0.f; B_[k + 3] = on ? b4.w : 0.f;
-        C_[k] = on ? c4.x : 0.f; C_[k + 1] = on ? c4.y : 0.f; C_[k + 2] = on ? c4.z : 0.f; C_[k + 3] = on ? c4.w : 0.f;
+        C_[k] = on ? c4.x * a.c_mult : 0.f; C_[k + 1] = on ? c4.y * a.c_mult : 0.f; C_[k + 2] = on ? c4.z * a.c_mult : 0.f; C_[k + 3] = on ? c4.w * a.c_mult : 0.f;
       }
     } else {
 #pragma unroll
@@ -303,7 +304,7 @@ template <int R, int K, bool VEC, int DEPTH, bool LOCAL> __global__ void __launc
         const int kk = k < nk ? k : 0;
         const float bv = xr[(nk ? bcol : inner) + kk], cv = xr[(nk ? ccol : inner) + kk];
         B_[k] = k < nk ? bv : 0.f;
-        C_[k] = k < nk ? cv : 0.f;
+        C_[k] = k < nk ? cv * a.c_mult : 0.f;
       }
     }
     g_.x = one_col ? 1.0f : xr[h * a.Pin + pc];
@@ -388,7 +389,7 @@ template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_b
         const int row = r0 + i;
         const float *xr = a.xbc + (size_t)row * a.C;
         if (j < N) v = xr[bcol + j];
-        else if (j < 2 * N) v = xr[ccol + j - N];
+        else if (j < 2 * N) v = xr[ccol + j - N] * a.c_mult;
         else if (j < 2 * N + P) v = j - 2 * N < a.Pin ? xr[h * a.Pin + j - 2 * N] : 1.0f;
         else v = a.steps[2 * ((size_t)row * a.heads + h) + (j - 2 * N - P)];
       }
@@ -1252,7 +1253,7 @@ extern "C" int mrs_hyb_conv_silu(const float *u, int ldu, const float *cw, const
 static int scan_launch(const float *xbc, const float *u, const float *dt_bias, const float *A_log, const float *D, const float *fixed_decay, float *state, float *out,
                        const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *steps, float *carry,
                        float *decay, int rows, int entries, int segments, int C, int ldu, int dt_col, int heads, int P, int N, int G, void *stream, int ones = 0,
-                       int ext_steps = 0) {
+                       int ext_steps = 0, float c_mult = 1.0f) {
   if (entries <= 0 || rows <= 0 || segments <= 0) return 0;
   if (heads <= 0 || G <= 0 || heads % G || P <= 0 || N <= 0) return fail("mrs_hyb_ssd_scan: bad head / group sizes");
   if (segments > 65535 || entries > 65535) return fail("mrs_hyb_ssd_scan: more than 65535 segments in one step");
@@ -1260,7 +1261,7 @@ static int scan_launch(const float *xbc, const float *u, const float *dt_bias, c
   const int Pin = P;  // value columns the rows carry; the state has `ones` more
   P += ones ? 1 : 0;
   ScanArgs a{xbc, u, dt_bias, A_log, D, fixed_decay, steps, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, decay, C, ldu, dt_col, heads, P, N, G, rows,
-             Pin, ext_steps ? 1 : 0};
+             Pin, ext_steps ? 1 : 0, c_mult};
   const bool vec = C % 4 == 0 && (heads * Pin) % 4 == 0 && N % 4 == 0 && ((uintptr_t)xbc % 16) == 0;
   const bool single = rows == segments;  // one row per segment (decode steps): no ring, step sizes inline
   if (!single && !ext_steps) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
@@ -1316,14 +1317,15 @@ extern "C" int mrs_hyb_decay_scan(const float *xkq, int ld, const float *fixed_d
 
 /* The same recurrence with step values the caller computed: steps [rows, heads, 2] = (what the state takes in, what it keeps) per row and head, S <- keep S + take k v^T,
  * o = S^T q; xkq [rows, ld] holds v [heads * P] | k [G * N] | q [G * N] from column 0.  ones != 0: the state has one more column per head that takes v = 1 (the running sum
- * of take * k beside the outer products): state [slots, heads, N, P + 1], out [rows, heads * (P + 1)], the last value of every head being that column's read-out. */
+ * of take * k beside the outer products): state [slots, heads, N, P + 1], out [rows, heads * (P + 1)], the last value of every head being that column's read-out.
+ * q_mult: the queries are multiplied by it as they are read. */
 extern "C" int mrs_hyb_gated_scan(const float *xkq, int ld, float *steps, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry,
                                   const int *seg_row0, const int *seg_len, const int *ent_seg0, float *carry, float *decay, int rows, int entries, int segments,
-                                  int heads, int P, int N, int G, int ones, void *stream) {
+                                  int heads, int P, int N, int G, int ones, float q_mult, void *stream) {
   if (!steps) return fail("mrs_hyb_gated_scan: the rows' step values are needed");
   if (ld < heads * P + 2 * G * N) return fail("mrs_hyb_gated_scan: rows shorter than v | k | q");
   return scan_launch(xkq, nullptr, nullptr, nullptr, nullptr, nullptr, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, steps, carry, decay, rows,
-                     entries, segments, ld, 0, 0, heads, P, N, G, stream, ones, 1);
+                     entries, segments, ld, 0, 0, heads, P, N, G, stream, ones, 1, q_mult);
 }
 
 static int qk_launch(const float *qkv, int ld, const float *qw, const float *kw, const float *freq, const int *tok_pos, const long long *slot_mapping, void *q_out,

@@ -35,6 +35,22 @@ __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v));
 __device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
 __device__ __forceinline__ float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
+// Sum over groups of R consecutive lanes (R = 4 or 16, groups aligned to R) with data-parallel-primitive moves: each step is one add whose second operand comes from another
+// lane of the same row of 16 (quad permutations, rotations inside the row) -- no trip through the LDS crossbar on the serial chain of a recurrence.
+template <int CTRL> __device__ __forceinline__ float dpp_add(float x) {
+  return x + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+template <int R> __device__ __forceinline__ float group_sum(float x) {
+  static_assert(R == 4 || R == 16, "groups of 4 or 16 lanes");
+  x = dpp_add<0xB1>(x);               // quad_perm [1, 0, 3, 2]
+  x = dpp_add<0x4E>(x);               // quad_perm [2, 3, 0, 1]
+  if (R == 16) {
+    x = dpp_add<0x124>(x);            // row_ror 4
+    x = dpp_add<0x128>(x);            // row_ror 8
+  }
+  return x;
+}
+
 // ---------------------------------------------------------------------------------- x / rms(x) times two weights
 template <class T> __global__ void __launch_bounds__(256) rmsnorm_pair_kernel(const float *__restrict__ x, int ldx, const float *__restrict__ w1, const float *__restrict__ w2,
                                                                                T *__restrict__ out1, T *__restrict__ out2, float *__restrict__ out2_32, int W, float eps, int one_plus) {
@@ -88,7 +104,7 @@ struct DeltaArgs {
   const int *seq_start, *seq_pos0, *seq_slot;
   int ldc, H, G, D, Dv, per;
 };
-template <int R, int K, bool VEC, int TC, int MAXC> __global__ void __launch_bounds__(512) delta_scan_kernel(DeltaArgs a, int rowpad) {
+template <int R, int K, bool VEC, int MAXREG> __global__ void __launch_bounds__(512) delta_scan_kernel(DeltaArgs a, int rowpad, int TC) {
   extern __shared__ __attribute__((aligned(16))) float sm[];  // [2][TC][rowpad]: k [D] | q [D] | decay [per] (padded to 4) | v [Dv] | beta
   constexpr int PT = 64 / R;
   const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, r = lane % R, p = (blockIdx.x * (nthr >> 6) + wave) * PT + lane / R;
@@ -107,33 +123,68 @@ template <int R, int K, bool VEC, int TC, int MAXC> __global__ void __launch_bou
   for (int k = 0; k < K; ++k) S[k] = (k < nk && carried) ? st[(size_t)(r * K + k) * Dv + pc] : 0.f;
   const int perp = (per + 3) & ~3, o_q = D, o_g = 2 * D, o_v = 2 * D + perp, o_b = o_v + Dv, rowlen = o_b + 1, stage = TC * rowpad;
   const int qcol = g * D, kcol = a.G * D + g * D, vcol = 2 * a.G * D + h * Dv;
-  float stg[TC][MAXC];
+  // this lane's operands of one staged row: k, decay and q of its K state rows (zeros / ones past the key size), the column's value and the write strength
+  constexpr bool PREFETCH = K <= 16;
+  const int base = nk ? r * K : 0;
+  auto ops = [&](const float *row, float *kv, float *gv, float *qv, float *sv) {
+    sv[0] = row[o_v + pc];
+    sv[1] = row[o_b];
+    const float g1 = row[o_g];
+    if (VEC) {
+#pragma unroll
+      for (int k = 0; k < K; k += 4) {
+        const int kk = base + (k < nk ? k : 0);
+        const float4 k4 = *(const float4 *)(row + kk), q4 = *(const float4 *)(row + o_q + kk);
+        float4 g4 = make_float4(g1, g1, g1, g1);
+        if (per > 1) g4 = *(const float4 *)(row + o_g + kk);
+        const bool on = k < nk;
+        kv[k] = on ? k4.x : 0.f; kv[k + 1] = on ? k4.y : 0.f; kv[k + 2] = on ? k4.z : 0.f; kv[k + 3] = on ? k4.w : 0.f;
+        qv[k] = on ? q4.x : 0.f; qv[k + 1] = on ? q4.y : 0.f; qv[k + 2] = on ? q4.z : 0.f; qv[k + 3] = on ? q4.w : 0.f;
+        gv[k] = g4.x; gv[k + 1] = g4.y; gv[k + 2] = g4.z; gv[k + 3] = g4.w;
+      }
+    } else {
+#pragma unroll
+      for (int k = 0; k < K; ++k) {
+        const int kk = k < nk ? base + k : 0;
+        kv[k] = k < nk ? row[kk] : 0.f;
+        qv[k] = k < nk ? row[o_q + kk] : 0.f;
+        gv[k] = per > 1 ? row[o_g + kk] : g1;
+      }
+    }
+  };
+  // a stage = TC rows of rowpad values, dealt to the threads flat: element e = tid + m nthr (m < MAXREG) is value e % rowpad of row e / rowpad.  Where an element comes from
+  // (its place in the first stage and how far one row moves it) is worked out once; a stage's loads are then one compare and one address each.
+  float stg[MAXREG];
+  const float *src[MAXREG];
+  int rstride[MAXREG], irow[MAXREG];
+  const int stage_n = TC * rowpad;
+#pragma unroll
+  for (int m = 0; m < MAXREG; ++m) {
+    const int e = tid + m * nthr;
+    src[m] = nullptr;
+    rstride[m] = 0;
+    irow[m] = 0;
+    if (e < stage_n) {
+      const int i = e / rowpad, j = e - i * rowpad;
+      irow[m] = i;
+      const size_t row = (size_t)r0 + i;
+      if (j < o_q) { src[m] = a.c + row * a.ldc + kcol + j; rstride[m] = a.ldc; }
+      else if (j < o_g) { src[m] = a.c + row * a.ldc + qcol + j - o_q; rstride[m] = a.ldc; }
+      else if (j < o_v) { if (j - o_g < per) { src[m] = a.dec + (row * a.H + h) * per + j - o_g; rstride[m] = a.H * per; } }
+      else if (j < o_b) { src[m] = a.c + row * a.ldc + vcol + j - o_v; rstride[m] = a.ldc; }
+      else if (j < rowlen) { src[m] = a.beta + row * a.H + h; rstride[m] = a.H; }
+    }
+  }
   auto fetch = [&](int c0) {
 #pragma unroll
-    for (int i = 0; i < TC; ++i)
-#pragma unroll
-      for (int m = 0; m < MAXC; ++m) {
-        const int j = tid + m * nthr, row = r0 + c0 + i;
-        float v = 0.f;
-        if (c0 + i < len && j < rowlen) {
-          const float *cr = a.c + (size_t)row * a.ldc;
-          if (j < o_q) v = cr[kcol + j];
-          else if (j < o_g) v = cr[qcol + j - o_q];
-          else if (j < o_v) v = j - o_g < per ? a.dec[((size_t)row * a.H + h) * per + j - o_g] : 0.f;
-          else if (j < o_b) v = cr[vcol + j - o_v];
-          else v = a.beta[(size_t)row * a.H + h];
-        }
-        stg[i][m] = v;
-      }
+    for (int m = 0; m < MAXREG; ++m) stg[m] = (src[m] && c0 + irow[m] < len) ? src[m][(size_t)c0 * rstride[m]] : 0.f;
   };
   auto put = [&](float *buf) {
 #pragma unroll
-    for (int i = 0; i < TC; ++i)
-#pragma unroll
-      for (int m = 0; m < MAXC; ++m) {
-        const int j = tid + m * nthr;
-        if (j < rowpad) buf[i * rowpad + j] = stg[i][m];
-      }
+    for (int m = 0; m < MAXREG; ++m) {
+      const int e = tid + m * nthr;
+      if (e < stage_n) buf[e] = stg[m];
+    }
   };
   fetch(0);
   put(sm);
@@ -144,64 +195,52 @@ template <int R, int K, bool VEC, int TC, int MAXC> __global__ void __launch_bou
     const bool more = c0 + TC < len;
     if (more) fetch(c0 + TC);
     const int cnt = len - c0 < TC ? len - c0 : TC;
-    for (int i = 0; i < cnt; ++i) {
-      const float *row = cur + i * rowpad;
-      const float vp = row[o_v + pc], be = row[o_b], g1 = row[o_g];
-      const int base = nk ? r * K : 0;
-      float acc = 0.f;
-      if (VEC) {
+    // a row's operands leave LDS one row ahead of their use (they do not depend on the state), into one of two register sets in turn: the serial chain per row is the
+    // two sums and the write between them
+    float ka[K], ga[K], qa[K], kb[K], gb[K], qb[K], sa[2], sb[2];
+    float *op = a.out + (size_t)(r0 + c0) * a.H * Dv + (size_t)h * Dv + pc;
+    const size_t ostep = (size_t)a.H * Dv;
+    auto step = [&](const float *kc, const float *gc, const float *qc, const float *sc) {
+      float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
-        for (int k = 0; k < K; k += 4) {
-          const int kk = base + (k < nk ? k : 0);
-          const float4 k4 = *(const float4 *)(row + kk);
-          float4 g4 = make_float4(g1, g1, g1, g1);
-          if (per > 1) g4 = *(const float4 *)(row + o_g + kk);
-          const bool on = k < nk;
-          const float kv[4] = {on ? k4.x : 0.f, on ? k4.y : 0.f, on ? k4.z : 0.f, on ? k4.w : 0.f}, gv[4] = {g4.x, g4.y, g4.z, g4.w};
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            S[k + q] *= gv[q];
-            acc = fmaf(S[k + q], kv[q], acc);
-          }
-        }
-      } else {
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-          const int kk = k < nk ? base + k : 0;
-          const float kv = k < nk ? row[kk] : 0.f, gv = per > 1 ? row[o_g + kk] : g1;
-          S[k] *= gv;
-          acc = fmaf(S[k], kv, acc);
+      for (int k = 0; k < K; k += 2) {
+        S[k] *= gc[k];
+        acc0 = fmaf(S[k], kc[k], acc0);
+        if (k + 1 < K) {
+          S[k + 1] *= gc[k + 1];
+          acc1 = fmaf(S[k + 1], kc[k + 1], acc1);
         }
       }
+      const float uw = sc[1] * (sc[0] - group_sum<R>(acc0 + acc1));
+      float o0 = 0.f, o1 = 0.f;
 #pragma unroll
-      for (int m = 1; m < R; m <<= 1) acc += __shfl_xor(acc, m, 64);
-      const float uw = be * (vp - acc);
-      float o = 0.f;
-      if (VEC) {
-#pragma unroll
-        for (int k = 0; k < K; k += 4) {
-          const int kk = base + (k < nk ? k : 0);
-          const float4 k4 = *(const float4 *)(row + kk), q4 = *(const float4 *)(row + o_q + kk);
-          const bool on = k < nk;
-          const float kv[4] = {on ? k4.x : 0.f, on ? k4.y : 0.f, on ? k4.z : 0.f, on ? k4.w : 0.f}, qv[4] = {on ? q4.x : 0.f, on ? q4.y : 0.f, on ? q4.z : 0.f, on ? q4.w : 0.f};
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            S[k + q] = fmaf(kv[q], uw, S[k + q]);
-            o = fmaf(S[k + q], qv[q], o);
-          }
-        }
-      } else {
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-          const int kk = k < nk ? base + k : 0;
-          const float kv = k < nk ? row[kk] : 0.f, qv = k < nk ? row[o_q + kk] : 0.f;
-          S[k] = fmaf(kv, uw, S[k]);
-          o = fmaf(S[k], qv, o);
+      for (int k = 0; k < K; k += 2) {
+        S[k] = fmaf(kc[k], uw, S[k]);
+        o0 = fmaf(S[k], qc[k], o0);
+        if (k + 1 < K) {
+          S[k + 1] = fmaf(kc[k + 1], uw, S[k + 1]);
+          o1 = fmaf(S[k + 1], qc[k + 1], o1);
         }
       }
-#pragma unroll
-      for (int m = 1; m < R; m <<= 1) o += __shfl_xor(o, m, 64);
-      if (r == 0 && live) a.out[(size_t)(r0 + c0 + i) * a.H * Dv + (size_t)h * Dv + p] = o;
+      const float o = group_sum<R>(o0 + o1);
+      if (r == 0 && live) *op = o;
+      op += ostep;
+    };
+    if (PREFETCH) {
+      ops(cur, ka, ga, qa, sa);
+      for (int i = 0; i < cnt; i += 2) {
+        if (i + 1 < cnt) ops(cur + (i + 1) * rowpad, kb, gb, qb, sb);
+        step(ka, ga, qa, sa);
+        if (i + 1 < cnt) {
+          if (i + 2 < cnt) ops(cur + (i + 2) * rowpad, ka, ga, qa, sa);
+          step(kb, gb, qb, sb);
+        }
+      }
+    } else {
+      for (int i = 0; i < cnt; ++i) {
+        ops(cur + i * rowpad, ka, ga, qa, sa);
+        step(ka, ga, qa, sa);
+      }
     }
     if (more) put(sm + (flip ^ 1) * stage);
     __syncthreads();
@@ -213,49 +252,99 @@ template <int R, int K, bool VEC, int TC, int MAXC> __global__ void __launch_bou
 }
 
 // ---------------------------------------------------------------------------------- exponential gates with a running stabiliser
-// u [rows, ldu]: raw input-gate logits at i_col + h, forget-gate logits at f_col + h, queries [H * D] at q_col (multiplied by q_mult in place).
+// u [rows, ldu]: raw input-gate logits at i_col + h, forget-gate logits at f_col + h.
 //   i = cap tanh((raw_i + bi) / cap);  f = logsigmoid(cap tanh((raw_f + bf) / cap));  m' = max(f + m, i)   (m carried per slot and head, 0 for a fresh sequence)
 //   steps [rows, H, 2] = (e^{i - m'}, e^{f + m - m'}): what the state takes in and what it keeps;  mexp [rows, H] = e^{-m'}
-// One workgroup per entry: the log gates of all its rows in parallel, then the maximum chain (one thread per head, two operations per row), then the exponentials in parallel.
-__global__ void __launch_bounds__(256) exp_gates_kernel(float *__restrict__ u, int ldu, int i_col, int f_col, int q_col, int nq, float q_mult, const float *__restrict__ bi,
-                                                        const float *__restrict__ bf, float cap, float *__restrict__ m_state, float *__restrict__ steps, float *__restrict__ mbuf,
-                                                        float *__restrict__ mexp, const int *__restrict__ seq_start, const int *__restrict__ seq_pos0,
-                                                        const int *__restrict__ seq_slot, int H) {
+// The chain m' = max(f + m, i) composes: a run of rows acts as m -> max(m + F, I) with F = sum f and I = the chain's result from minus infinity.  An entry's rows are cut
+// into 256 / H pieces; every (piece, head) thread folds its piece, one thread per head chains the pieces, then every thread replays its piece from the right start.
+// mbuf [rows + entries, H]: m' of every row, then the m every entry started from.
+__device__ __forceinline__ void log_gates(const float *ur, int i_col, int f_col, int h, const float *bi, const float *bf, float cap, float &ig, float &fg) {
+  ig = cap * tanhf((ur[i_col + h] + bi[h]) / cap);
+  fg = -softplus_f(-(cap * tanhf((ur[f_col + h] + bf[h]) / cap)));
+}
+__global__ void __launch_bounds__(256) exp_gates_log_kernel(const float *__restrict__ u, int ldu, int i_col, int f_col, const float *__restrict__ bi, const float *__restrict__ bf,
+                                                            float cap, float *__restrict__ steps, int H, int n) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= n) return;
+  float ig, fg;
+  log_gates(u + (size_t)(e / H) * ldu, i_col, f_col, e % H, bi, bf, cap, ig, fg);
+  steps[2 * (size_t)e] = ig;
+  steps[2 * (size_t)e + 1] = fg;
+}
+// one workgroup per entry.  FUSED (steps of single rows): the log gates before and the exponentials after the chain in the same launch.
+template <bool FUSED> __global__ void __launch_bounds__(256) exp_gates_chain_kernel(const float *__restrict__ u, int ldu, int i_col, int f_col, const float *__restrict__ bi,
+                                                                                    const float *__restrict__ bf, float cap, float *__restrict__ m_state, float *__restrict__ steps,
+                                                                                    float *__restrict__ mbuf, float *__restrict__ mexp, const int *__restrict__ seq_start,
+                                                                                    const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot, int H, int rows) {
+  __shared__ float pF[256], pI[256], pM[256];
   const int s = blockIdx.x, r0 = seq_start[s], len = seq_start[s + 1] - r0;
   if (len <= 0) return;
-  for (int e = threadIdx.x; e < len * H; e += 256) {
-    const int t = r0 + e / H, h = e % H;
-    const float *ur = u + (size_t)t * ldu;
-    const float ig = cap * tanhf((ur[i_col + h] + bi[h]) / cap), fr = cap * tanhf((ur[f_col + h] + bf[h]) / cap);
-    steps[2 * ((size_t)t * H + h)] = ig;
-    steps[2 * ((size_t)t * H + h) + 1] = -softplus_f(-fr);
+  if (FUSED) {
+    for (int e = threadIdx.x; e < len * H; e += 256) {
+      float ig, fg;
+      log_gates(u + (size_t)(r0 + e / H) * ldu, i_col, f_col, e % H, bi, bf, cap, ig, fg);
+      steps[2 * ((size_t)r0 * H + e)] = ig;
+      steps[2 * ((size_t)r0 * H + e) + 1] = fg;
+    }
+    __syncthreads();
   }
-  if (q_mult != 1.0f)
-    for (size_t e = threadIdx.x; e < (size_t)len * nq; e += 256) u[(size_t)(r0 + e / nq) * ldu + q_col + e % nq] *= q_mult;
-  __syncthreads();
   float *ms = m_state + (size_t)seq_slot[s] * H;
   const bool carried = seq_pos0[s] > 0;
+  const int pieces = 256 / H, per = (len + pieces - 1) / pieces;
+  const int pc = threadIdx.x / H, ph = threadIdx.x % H;
+  const int i0 = pc * per, i1 = (i0 + per < len) ? i0 + per : len;
+  const bool mine = pc < pieces && i0 < len;
+  if (mine) {
+    float F = 0.f, I = -FLT_MAX;
+    for (int i = i0; i < i1; ++i) {
+      const float *g = steps + 2 * ((size_t)(r0 + i) * H + ph);
+      F += g[1];
+      I = fmaxf(I + g[1], g[0]);
+    }
+    pF[threadIdx.x] = F;
+    pI[threadIdx.x] = I;
+  }
+  __syncthreads();
   if (threadIdx.x < H) {
-    const int h = threadIdx.x;
-    float m = carried ? ms[h] : 0.f;
-    for (int i = 0; i < len; ++i) {
-      const float *g = steps + 2 * ((size_t)(r0 + i) * H + h);
+    float m = carried ? ms[threadIdx.x] : 0.f;
+    mbuf[((size_t)rows + s) * H + threadIdx.x] = m;
+    for (int c = 0; c < pieces && c * per < len; ++c) {
+      pM[c * H + threadIdx.x] = m;
+      m = fmaxf(m + pF[c * H + threadIdx.x], pI[c * H + threadIdx.x]);
+    }
+    ms[threadIdx.x] = m;   // the entry's last m'
+  }
+  __syncthreads();
+  if (mine) {
+    float m = pM[threadIdx.x];
+    for (int i = i0; i < i1; ++i) {
+      const float *g = steps + 2 * ((size_t)(r0 + i) * H + ph);
       m = fmaxf(g[1] + m, g[0]);
-      mbuf[(size_t)(r0 + i) * H + h] = m;
+      mbuf[(size_t)(r0 + i) * H + ph] = m;
     }
   }
+  if (!FUSED) return;
   __syncthreads();
   for (int e = threadIdx.x; e < len * H; e += 256) {
     const int i = e / H, h = e % H, t = r0 + i;
-    const float m_old = i ? mbuf[(size_t)(t - 1) * H + h] : (carried ? ms[h] : 0.f), m_new = mbuf[(size_t)t * H + h];
+    const float m_old = i ? mbuf[(size_t)(t - 1) * H + h] : mbuf[((size_t)rows + s) * H + h], m_new = mbuf[(size_t)t * H + h];
     float *g = steps + 2 * ((size_t)t * H + h);
     const float ig = g[0], fg = g[1];
     g[0] = expf(ig - m_new);
     g[1] = expf(fg + m_old - m_new);
     mexp[(size_t)t * H + h] = expf(-m_new);
   }
-  __syncthreads();   // every m_old has been read
-  if (threadIdx.x < H) ms[threadIdx.x] = mbuf[(size_t)(r0 + len - 1) * H + threadIdx.x];
+}
+__global__ void __launch_bounds__(256) exp_gates_exp_kernel(float *__restrict__ steps, const float *__restrict__ mbuf, float *__restrict__ mexp, const int *__restrict__ tok_seq,
+                                                            const int *__restrict__ seq_start, int H, int rows) {
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= rows * H) return;
+  const int t = e / H, h = e % H, s = tok_seq[t];
+  const float m_old = t > seq_start[s] ? mbuf[(size_t)(t - 1) * H + h] : mbuf[((size_t)rows + s) * H + h], m_new = mbuf[(size_t)e];
+  const float ig = steps[2 * (size_t)e], fg = steps[2 * (size_t)e + 1];
+  steps[2 * (size_t)e] = expf(ig - m_new);
+  steps[2 * (size_t)e + 1] = expf(fg + m_old - m_new);
+  mexp[e] = expf(-m_new);
 }
 
 // ---------------------------------------------------------------------------------- per-head output norm with a gate
@@ -353,20 +442,23 @@ extern "C" int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, co
   if (ldc < 2 * G * D + H * Dv) return fail("mrs_hyb_delta_scan: rows shorter than q | k | v");
   DeltaArgs a{c, beta, dec, state, out, seq_start, seq_pos0, seq_slot, ldc, H, G, D, Dv, per};
   int R = lanes_per_column;
-  if (R != 4 && R != 16) R = ((long long)entries * H * ((Dv + 15) / 16) >= 1024 || D < 64) ? 4 : 16;
+  if (R != 4 && R != 16) R = ((long long)entries * H * ((Dv + 15) / 16) >= 2048 || D < 64) ? 4 : 16;
   const int PT = 64 / R;
   const int perp = (per + 3) & ~3, rowlen = 2 * D + perp + Dv + 1, rowpad = (rowlen + 3) & ~3;
-  constexpr int TC = 4, MAXC = 8;
-  const int nw_all = (Dv + PT - 1) / PT, nw_stage = (rowpad + MAXC * 64 - 1) / (MAXC * 64);  // waves for the columns; waves whose registers can stage a row of operands
-  int nw = nw_all > 8 ? 8 : nw_all;
+  constexpr int MAXREG = 12, TC_MAX = 16;
+  // waves for the columns; waves whose registers can stage eight rows of operands at a time (a stage must outlast the latency of the loads for the next one)
+  const int nw_all = (Dv + PT - 1) / PT, nw_stage = (8 * rowpad + MAXREG * 64 - 1) / (MAXREG * 64);
+  int nw = nw_all > 8 ? 8 : nw_all;   // (four-wave workgroups, one chain per SIMD, measured no faster: the chain is bound by its own instruction count)
   const int nblk = (nw_all + nw - 1) / nw;
-  if (nw < nw_stage) nw = nw_stage;  // few value columns next to long keys: further waves only help to stage (their columns lie past Dv and are never written)
-  if (nw > 8) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers");
+  if (nw < nw_stage) nw = nw_stage > 8 ? 8 : nw_stage;  // few value columns next to long keys: further waves only help to stage (their columns lie past Dv and are never written)
+  int TC = (MAXREG * 64 * nw) / rowpad;
+  TC = TC > TC_MAX ? TC_MAX : TC;
+  if (TC > 65536 / (8 * rowpad)) TC = 65536 / (8 * rowpad);
+  if (TC < 1) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers / 64 KB of LDS");
   const size_t lds = (size_t)2 * TC * rowpad * 4;
-  if (lds > 65536) return fail("mrs_hyb_delta_scan: staged rows above 64 KB");
   const bool vec = D % 4 == 0;
   dim3 grid(nblk, H, entries), block(64 * nw);
-#define MRS_DELTA_(R_, K_, V_) hipLaunchKernelGGL((delta_scan_kernel<R_, K_, V_, TC, MAXC>), grid, block, lds, S_(stream), a, rowpad)
+#define MRS_DELTA_(R_, K_, V_) hipLaunchKernelGGL((delta_scan_kernel<R_, K_, V_, MAXREG>), grid, block, lds, S_(stream), a, rowpad, TC)
 #define MRS_DELTA(R_, K_) do { if (vec) MRS_DELTA_(R_, K_, true); else MRS_DELTA_(R_, K_, false); } while (0)
   if (R == 4) {
     if (D <= 32) MRS_DELTA(4, 8); else if (D <= 64) MRS_DELTA(4, 16); else if (D <= 128) MRS_DELTA(4, 32); else MRS_DELTA(4, 64);
@@ -378,13 +470,22 @@ extern "C" int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, co
   return ok_or("mrs_hyb_delta_scan");
 }
 
-/* steps [rows, H, 2], mbuf [rows, H] (scratch), mexp [rows, H]; m_state [slots, H]; the query columns of u are multiplied by q_mult in place */
-extern "C" int mrs_hyb_exp_gates(float *u, int ldu, int i_col, int f_col, int q_col, int nq, float q_mult, const float *bi, const float *bf, float cap, float *m_state,
-                                 float *steps, float *mbuf, float *mexp, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, void *stream) {
+/* steps [rows, H, 2], mbuf [rows + entries, H] (scratch), mexp [rows, H]; m_state [slots, H].  Steps of single rows run one launch, steps with portions three (the log
+ * gates and the exponentials of all rows in parallel around the per-entry chain). */
+extern "C" int mrs_hyb_exp_gates(const float *u, int ldu, int i_col, int f_col, const float *bi, const float *bf, float cap, float *m_state, float *steps, float *mbuf,
+                                 float *mexp, const int *tok_seq, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, void *stream) {
   if (rows <= 0 || entries <= 0) return 0;
   if (H <= 0 || H > 256 || !(cap > 0.f)) return fail("mrs_hyb_exp_gates: 1 .. 256 heads, a positive gate cap");
-  hipLaunchKernelGGL(exp_gates_kernel, dim3(entries), dim3(256), 0, S_(stream), u, ldu, i_col, f_col, q_col, nq, q_mult, bi, bf, cap, m_state, steps, mbuf, mexp, seq_start,
-                     seq_pos0, seq_slot, H);
+  if (rows == entries) {
+    hipLaunchKernelGGL(exp_gates_chain_kernel<true>, dim3(entries), dim3(256), 0, S_(stream), u, ldu, i_col, f_col, bi, bf, cap, m_state, steps, mbuf, mexp, seq_start, seq_pos0,
+                       seq_slot, H, rows);
+    return ok_or("mrs_hyb_exp_gates");
+  }
+  const int n = rows * H;
+  hipLaunchKernelGGL(exp_gates_log_kernel, dim3((n + 255) / 256), dim3(256), 0, S_(stream), u, ldu, i_col, f_col, bi, bf, cap, steps, H, n);
+  hipLaunchKernelGGL(exp_gates_chain_kernel<false>, dim3(entries), dim3(256), 0, S_(stream), u, ldu, i_col, f_col, bi, bf, cap, m_state, steps, mbuf, mexp, seq_start, seq_pos0,
+                     seq_slot, H, rows);
+  hipLaunchKernelGGL(exp_gates_exp_kernel, dim3((n + 255) / 256), dim3(256), 0, S_(stream), steps, mbuf, mexp, tok_seq, seq_start, H, rows);
   return ok_or("mrs_hyb_exp_gates");
 }
 

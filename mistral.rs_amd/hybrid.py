@@ -59,14 +59,14 @@ _SIGS = {
     "mrs_hyb_layernorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _vp],
     "mrs_hyb_qkv_bias_temp_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i, _vp],
     "mrs_hyb_paged_talk_sigmoid_attn": [_vp] * 9 + [_i, _vp] + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _vp, _i, _vp],
-    "mrs_hyb_gated_scan": [_vp, _i] + [_vp] * 11 + [_i] * 8 + [_vp],
+    "mrs_hyb_gated_scan": [_vp, _i] + [_vp] * 11 + [_i] * 8 + [_f, _vp],
     "mrs_hyb_qk_headnorm_rope_cache": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _f, _i, _vp],
     "mrs_hyb_paged_attn_chunked": [_vp] * 7 + [_i] * 8 + [_f, _i, _vp, _vp, _vp, _i, _i, _f, _i, _vp, _vp, _i, _i, _vp, _i, _vp],
     "mrs_hyb_route_topk_softmax": [_vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _vp],
     "mrs_hyb_rmsnorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
     "mrs_hyb_delta_prep": [_vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "mrs_hyb_delta_scan": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 8 + [_vp],
-    "mrs_hyb_exp_gates": [_vp, _i, _i, _i, _i, _i, _f, _vp, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "mrs_hyb_exp_gates": [_vp, _i, _i, _i, _vp, _vp, _f] + [_vp] * 8 + [_i, _i, _i, _vp],
     "mrs_hyb_head_norm_gate": [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _vp],
     "mrs_hyb_norm_pair_add": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _i, _vp],
     "mrs_hyb_round_cols": [_vp, _i, _vp, _i, _i, _i, _vp],
@@ -678,8 +678,7 @@ class WindowAttention(_Module):
         if s.chunk or s.sink or s.head_gate:
             if s.window or s.keep_first:
                 raise NotImplementedError("a learned sink / a per-head gate beside a sliding window")
-            # a chunk holds few keys: no key splits (unchunked layers of single-row steps may split)
-            scratch, splits = (None, 0) if s.chunk else m.key_splits(b, s.heads, s.vdim)
+            scratch, splits = m.key_splits(b, s.heads, s.vdim, s.chunk)   # single-row steps deal a long chunk's keys to several workgroups
             _call("mrs_hyb_paged_attn_chunked", q, self.k_cache, self.v_cache, b.block_tables, b.tok_seq, b.tok_pos, o, T, s.heads, s.kv_heads, s.dim, s.vdim, m.block_size,
                   b.max_blocks, s.chunk, s.scale, m.dt, b.seg_entry, b.seg_row0, b.seg_len, b.segments, RaggedBatch.SEGMENT, 0.0, int(s.sink), self.sink,
                   qkv[:, self.gate_col:] if s.head_gate else None, qkv.stride(0), 1, scratch, splits)
@@ -1201,7 +1200,7 @@ class DeltaRuleMixer(_Module):
 
 
 class MlstmMixer(_Module):
-    """v | k | q | gate | input-gate | forget-gate logits in one product; q times dim^(-1/2); log gates i = cap tanh((.. + b) / cap), f = logsigmoid(cap tanh((.. + b) /
+    """v | k | q | gate | input-gate | forget-gate logits in one product; q times dim^(-1/2) (as the scan reads it); log gates i = cap tanh((.. + b) / cap), f = logsigmoid(cap tanh((.. + b) /
     cap)); with the running maximum m' = max(f + m, i) (m starts at 0): S <- e^{f + m - m'} S + e^{i - m'} k v^T, n likewise with k alone, o = S^T q / (max(|n . q|,
     e^{-m'}) + 1e-6).  n rides as one more column of the state (a value that is always 1), so the recurrence is the gated scan of the state-space mixers with step values
     from the gates: portions run their segments in parallel.  o / rms(o) per head, times `norm` [heads * vdim], times sigmoid(gate), output projection.  Carries S | n
@@ -1241,9 +1240,9 @@ class MlstmMixer(_Module):
         f32 = dict(dtype=torch.float32, device=dev)
         u = m.linear(h, self.w_in)                                          # f32 [T, v | k | q | gate | i | f]
         steps = torch.empty(T, s.heads, 2, **f32)
-        mbuf, mexp = torch.empty(T, s.heads, **f32), torch.empty(T, s.heads, **f32)
-        _call("mrs_hyb_exp_gates", u, u.stride(0), self.i_col, self.f_col, self.q_col, s.heads * s.dim, self.q_mult, self.bi, self.bf, s.gate_cap, self.m_state, steps, mbuf,
-              mexp, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, s.heads)
+        mbuf, mexp = torch.empty(T + b.entries, s.heads, **f32), torch.empty(T, s.heads, **f32)
+        _call("mrs_hyb_exp_gates", u, u.stride(0), self.i_col, self.f_col, self.bi, self.bf, s.gate_cap, self.m_state, steps, mbuf, mexp, b.tok_seq, b.seq_start, b.seq_pos0,
+              b.seq_slot, T, b.entries, s.heads)
         P = s.vdim + 1
         y = torch.empty(T, s.heads * P, **f32)
         carry = decay = None
@@ -1251,7 +1250,7 @@ class MlstmMixer(_Module):
             carry = torch.empty(b.segments, s.heads, s.dim, P, **f32)
             decay = torch.empty(b.segments, s.heads, **f32)
         _call("mrs_hyb_gated_scan", u, u.stride(0), steps, self.state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, carry, decay, T, b.entries,
-              b.segments, s.heads, s.vdim, s.dim, s.heads, 1)
+              b.segments, s.heads, s.vdim, s.dim, s.heads, 1, self.q_mult)
         o = torch.empty(T, s.heads * s.vdim, dtype=m.torch_dtype, device=dev)
         _call("mrs_hyb_head_norm_gate", y, P, mexp, self.norm, 1, u[:, self.g_col:], u.stride(0), 1, o, T, s.heads, s.vdim, m.spec.eps, m.dt)
         m.linear(o, self.w_o, out=x, accumulate=accumulate)
@@ -1462,12 +1461,13 @@ class HybridDecoder:
     KEYS_PER_SPLIT = 256   # at least this many keys (of the longest table in the batch) per workgroup
     KEY_SPLITS = 32
 
-    def key_splits(self, b: RaggedBatch, heads: int, vdim: int):
+    def key_splits(self, b: RaggedBatch, heads: int, vdim: int, most_keys: int = 0):
         """(scratch, splits) for an attention launch over unwindowed keys: a step in which every entry brings one row deals each row's keys to several workgroups
-        (one wave walking thousands of keys is latency-bound); (None, 0) otherwise."""
+        (one wave walking thousands of keys is latency-bound); (None, 0) otherwise.  most_keys > 0: no row reads more keys than that (a chunk, a window)."""
         if b.seg_rows != 1 or b.rows > self.KEY_SPLIT_ROWS:
             return None, 0
-        splits = min(self.KEY_SPLITS, (b.max_blocks * self.block_size) // self.KEYS_PER_SPLIT)
+        keys = b.max_blocks * self.block_size
+        splits = min(self.KEY_SPLITS, (min(keys, most_keys) if most_keys > 0 else keys) // self.KEYS_PER_SPLIT)
         if splits < 2:
             return None, 0
         return torch.empty(splits, b.rows, heads, vdim + 2, dtype=torch.float32, device=self.device), splits

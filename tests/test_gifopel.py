@@ -473,13 +473,12 @@ def test_exponential_gates_and_matrix_memory_over_segments_and_single_rows(dev, 
         b = _batch(dev, [(at[j], n, slots[j]) for j, n in parts])
         u = torch.cat([seqs[j][at[j]:at[j] + n] for j, n in parts]).to(dev)
         T = u.shape[0]
-        steps, mbuf, mexp = torch.empty(T, H, 2, device=dev), torch.empty(T, H, device=dev), torch.empty(T, H, device=dev)
-        _call("mrs_hyb_exp_gates", u, ld, i_col, f_col, q_col, nk, float(np.float32(D) ** np.float32(-0.5)), bi.to(dev), bf.to(dev), cap, m_state, steps, mbuf, mexp,
-              b.seq_start, b.seq_pos0, b.seq_slot, T, len(parts), H)
+        steps, mbuf, mexp = torch.empty(T, H, 2, device=dev), torch.empty(T + len(parts), H, device=dev), torch.empty(T, H, device=dev)
+        _call("mrs_hyb_exp_gates", u, ld, i_col, f_col, bi.to(dev), bf.to(dev), cap, m_state, steps, mbuf, mexp, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, T, len(parts), H)
         y = torch.empty(T, H * (Dv + 1), device=dev)
         carry, dk = torch.empty(b.segments, H, D, Dv + 1, device=dev), torch.empty(b.segments, H, device=dev)
         _call("mrs_hyb_gated_scan", u, ld, steps, state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, carry, dk, T, len(parts), b.segments,
-              H, Dv, D, H, 1)
+              H, Dv, D, H, 1, float(np.float32(D) ** np.float32(-0.5)))
         o = torch.empty(T, nv, device=dev)
         _call("mrs_hyb_head_norm_gate", y, Dv + 1, mexp, nw.to(dev), 1, u[:, g_col:], ld, 1, o, T, H, Dv, 1e-5, 2)
         r = 0
@@ -756,6 +755,23 @@ def test_slow_states_carry_the_first_tokens_across_a_long_prompt_and_decoding(de
     sv = Served(cfg, w, dev, max_tokens=448)
     got = sv.step([(1, t[:63])]) + sv.step([(1, t[63:65])]) + sv.step([(1, t[65:120])]) + [sv.step([(1, [x])])[0] for x in t[120:]]
     assert rel(torch.cat(got), want) < 5e-5
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("size", [0, 600, 300])
+def test_decoding_with_split_keys_inside_a_long_chunk(dev, size):
+    """single-row steps over hundreds of keys deal a row's keys to several workgroups (some shares empty right behind a chunk border); two sequences of unequal length"""
+    cfg = config([par(heads=4, kv_heads=2, dim=16, vdim=8, size=size, dims=8, scale=0.6, mlp=None)])
+    w = weights(cfg, 41)
+    wd = f64(w)
+    ta, tb = toks(640, cfg["vocab"], 42), toks(290, cfg["vocab"], 43)
+    wa, wb = logits_of(cfg, wd, ta), logits_of(cfg, wd, tb)
+    sv = Served(cfg, w, dev, max_tokens=1024)
+    sv.step([(1, ta[:590]), (2, tb[:240])])
+    assert sv.m.key_splits(_batch(dev, [(600, 1, 0)]), 4, 8, size)[1] >= 2 if size != 300 else True
+    for i in range(50):
+        ga, gb = sv.step([(1, [ta[590 + i]]), (2, [tb[240 + i]])])
+        assert rel(ga, wa[590 + i:591 + i]) < 3e-5 and rel(gb, wb[240 + i:241 + i]) < 3e-5, i
 
 
 @pytest.mark.gpu
