@@ -361,7 +361,7 @@ template <int R, int K, bool VEC, bool LOCAL, int NT> __global__ void __launch_b
   constexpr int TC = 8;  // rows per stage; a thread stages columns tid and tid + nthr of every row (16 registers)
   extern __shared__ __attribute__((aligned(16))) float sm[];  // [2][TC][rowpad]: B [N] | C [N] | x [P] | dt | decay
   constexpr int PT = 64 / R;
-  const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, r = lane % R, p = wave * PT + lane / R;
+  const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, r = lane % R, p = (blockIdx.x * (nthr >> 6) + wave) * PT + lane / R;
   const int h = blockIdx.y, z = blockIdx.z;
   const int s = a.seg_entry[z], r0 = a.seg_row0[z], len = a.seg_len[z];
   const bool first = z == a.ent_seg0[s], last = z == a.ent_seg0[s + 1] - 1;
@@ -1267,15 +1267,17 @@ static int scan_launch(const float *xbc, const float *u, const float *dt_bias, c
   if (!single && !ext_steps) hipLaunchKernelGGL(ssd_steps_kernel, dim3((rows * heads + 255) / 256), dim3(256), 0, S_(stream), a);
   const bool split = segments > entries;
 #define MRS_SCAN_(R, K, V, DP, L) hipLaunchKernelGGL((ssd_scan_kernel<R, K, V, DP, L>), dim3((P + 64 / R - 1) / (64 / R), heads, segments), dim3(64), 0, S_(stream), a)
-#define MRS_SCAN_LDS_(R, K, V, L) do { if (nw <= 4) hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 256>), dim3(1, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); \
-                                       else hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 1024>), dim3(1, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); } while (0)
-  // portions: the LDS-staged kernel when one workgroup can hold a head's P (<= 16 waves) and two columns per thread cover a staged row
-  int nw = 0;
+#define MRS_SCAN_LDS_(R, K, V, L) do { if (nw <= 4) hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 256>), dim3(nblk, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); \
+                                       else hipLaunchKernelGGL((ssd_scan_lds_kernel<R, K, V, L, 1024>), dim3(nblk, heads, segments), dim3(64 * nw), lds_bytes, S_(stream), a, rowpad); } while (0)
+  // portions: the LDS-staged kernel when two columns per thread cover a staged row; a head's P columns take workgroups of at most 16 waves (each stages the rows for itself)
+  int nw = 0, nblk = 1;
   const int rowpad = (2 * N + P + 2 + 3) & ~3;
   const size_t lds_bytes = (size_t)2 * 8 * rowpad * 4;
   auto plan_lds = [&](int R_) {
-    nw = (P + 64 / R_ - 1) / (64 / R_);
-    if (single || nw > 16 || rowpad > 2 * 64 * nw || lds_bytes > 65536) nw = 0;
+    const int all = (P + 64 / R_ - 1) / (64 / R_);
+    nblk = all <= 16 ? 1 : (all + 7) / 8;  // past one workgroup: pieces of at most eight waves, several of which fit a compute unit side by side
+    nw = (all + nblk - 1) / nblk;
+    if (single || rowpad > 2 * 64 * nw || lds_bytes > 65536) nw = 0;
   };
 #define MRS_SCAN(R, K, DP) do { \
     plan_lds(R); \
