@@ -1275,7 +1275,7 @@ static int scan_launch(const float *xbc, const float *u, const float *dt_bias, c
   const size_t lds_bytes = (size_t)2 * 8 * rowpad * 4;
   auto plan_lds = [&](int R_) {
     const int all = (P + 64 / R_ - 1) / (64 / R_);
-    nblk = all <= 16 ? 1 : (all + 7) / 8;  // past one workgroup: pieces of at most eight waves, several of which fit a compute unit side by side
+    nblk = (all + 15) / 16;
     nw = (all + nblk - 1) / nblk;
     if (single || rowpad > 2 * 64 * nw || lds_bytes > 65536) nw = 0;
   };
@@ -1287,6 +1287,8 @@ static int scan_launch(const float *xbc, const float *u, const float *dt_bias, c
     if (single) { if (vec) MRS_SCAN_(R, K, true, 1, false); else MRS_SCAN_(R, K, false, 1, false); } \
     else if (nw) { if (vec) MRS_SCAN_LDS_(R, K, true, false); else MRS_SCAN_LDS_(R, K, false, false); } \
     else { if (vec) MRS_SCAN_(R, K, true, DP, false); else MRS_SCAN_(R, K, false, DP, false); } } while (0)
+  // (a head whose columns need more than sixteen waves -- a value size of 256 and the column of ones -- runs as two workgroups that each stage the rows; two lanes per
+  // column with 64 state rows each, which would keep it in one, measured 1.8x slower, pieces of eight waves 1.1x slower)
   if (N <= 16) MRS_SCAN(2, 8, 8);
   else if (N <= 64) MRS_SCAN(4, 16, 6);
   else if (N <= 128) MRS_SCAN(4, 32, 4);

@@ -439,7 +439,7 @@ def test_delta_state_keeps_a_planted_pair_for_hundreds_of_rows_and_replaces_it(d
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,D,Dv,cap", [(2, 12, 16, 9.0), (3, 7, 5, 2.5), (1, 64, 64, 15.0), (4, 16, 127, 6.0), (2, 130, 8, 30.0)])
+@pytest.mark.parametrize("H,D,Dv,cap", [(2, 12, 16, 9.0), (3, 7, 5, 2.5), (1, 64, 64, 15.0), (4, 16, 127, 6.0), (2, 130, 8, 30.0), (2, 64, 256, 8.0), (1, 128, 300, 8.0), (1, 20, 257, 8.0)])
 def test_exponential_gates_and_matrix_memory_over_segments_and_single_rows(dev, H, D, Dv, cap):
     """gate kernel + gated scan with the normaliser column + head norm, two sequences through reused slots, portions longer than a segment (64 rows), a portion that ends a
     segment exactly, single rows: against the restatement's cell on the whole sequences"""
