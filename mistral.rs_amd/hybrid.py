@@ -1,8 +1,10 @@
-"""Layer-list ("hybrid") decoders served in their checkpoint dtype: every layer is `x += mixer(norm(x))` then optionally `x += feed_forward(norm(x))`, the mixer being
-one of the registered kinds (`MIXERS`: state-space-duality recurrence, paged softmax attention with a sliding window and kept first tokens, paged sigmoid attention with a
-distance bias and mixed head scores), the feed-forward one of `FEED_FORWARDS` (sigmoid-routed experts with a gated shared expert, softmax-routed clamped-GLU experts, a
-dense xIELU layer).  The norms are one-plus RMS norms before every sublayer, or layer norms with bias before AND after every sublayer (`HybridSpec.norm`, `post_norms`).
-The Gekilix and Sobunex architectures (config.json `"architecture"`) are two such lists.
+"""Layer-list ("hybrid") decoders served in their checkpoint dtype: every layer is `x += mixer(norm(x))` then optionally `x += feed_forward(norm(x))` (or both sublayers
+reading two norms of the same x: `parallel_sublayers`), the mixer being one of the registered kinds (`MIXERS`: state-space-duality recurrence, paged softmax attention with a
+sliding window / position chunks / kept first tokens / a learned sink, paged sigmoid attention with a distance bias and mixed head scores, sink attention with convolved
+projections, retention, latent attention, the gated delta rule, a matrix memory with exponential gates, two mixers side by side), the feed-forward one of `FEED_FORWARDS`
+(sigmoid-routed experts with a gated shared expert, softmax-routed clamped-GLU experts, routed squared-ReLU experts weighted over the chosen logits, dense xIELU and SiLU-GLU
+layers).  The norms are RMS norms (plain or one-plus weights) before every sublayer, or layer norms with bias before AND after every sublayer (`HybridSpec.norm`,
+`post_norms`).  The Gekilix, Sobunex, Setopel and Gifopel architectures (config.json `"architecture"`) are such lists.
 
 The step function is `HybridDecoder.forward_batch(batch)`: ONE ragged batch -- prompt portions of any length next to single decoded tokens -- through the HIP kernels of
 csrc/hyb_kernels.hip and csrc/hyb_gemm.hip (C ABI, this process's current stream; PyTorch owns buffers and the stream, nothing else).  What the sequences carry between
