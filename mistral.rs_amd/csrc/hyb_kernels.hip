@@ -5,6 +5,9 @@
 //   short causal convolution + SiLU with carried taps, the state-space-duality recurrence with a carried f32 state,
 //   whole-projection query / key norm + interleaved partial rotary + paged K / V write, paged attention with a sliding window and kept first tokens,
 //   sigmoid top-k routing, stable expert dispatch, scaled row gather, SiLU-GLU, weighted combine with a gated shared expert.
+//   Options that later designs added next to these: the recurrence with fixed decays or with step values from the caller and a column of ones, query / key norms per head,
+//   attention inside position chunks with a learned sink and one gate logit per head, a router bias with a softmax over the chosen logits (the delta-rule and
+//   exponential-gate kernels are in hyb_recur.hip).
 //
 // What is f32 regardless of the serving dtype: the residual stream, every norm, positions and angles, scores / softmax / the weighted value sum, router logits and
 // scores, decays, step sizes and the recurrent state.  T below is the dtype of GEMM operands and of the K / V pages: bf16, or f32 in the all-f32 mode.

@@ -1168,6 +1168,10 @@ class DeltaRuleMixer(_Module):
         self.g_col = self.a_col + want[4]
         self.w_a2 = self.w(get, p + "a2", True) if lowrank_a else None
         self.w_g2 = self.w(get, p + "g2", True) if lowrank_g else None
+        self.w_ag2 = None
+        if lowrank_a and lowrank_g:   # both second steps as ONE product on the adjacent first steps: a block-diagonal weight (the zeros add nothing, exactly)
+            self.w_ag2 = torch.zeros(ndec + self.nv, self.rank_a + self.rank_g, dtype=dt, device=dev)
+            self.w_ag2[:ndec, :self.rank_a], self.w_ag2[ndec:, self.rank_a:] = self.w_a2, self.w_g2
         self.conv_w = torch.cat([get(p + n + ".conv") for n in ("q", "k", "v")], 0).to(dev, torch.float32).contiguous()   # [channels, taps]
         self.A_log, self.dt_bias, self.norm = (self.w(get, p + n, False).reshape(-1) for n in ("A_log", "dt_bias", "norm"))
         self.w_o = self.w(get, p + "o", True)
@@ -1184,12 +1188,15 @@ class DeltaRuleMixer(_Module):
         c = torch.empty(T, self.channels, **f32)
         _call("mrs_hyb_conv", u, u.stride(0), None, self.conv_w, None, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, c, T, b.entries, self.channels,
               s.conv, 1)
-        a = u[:, self.a_col:]
-        if self.w_a2 is not None:                                           # the decay's second step: a product on the rounded first step
-            a = m.linear(m.round_cols(a, self.rank_a), self.w_a2)
-        gate = u[:, self.g_col:]
-        if self.w_g2 is not None:
-            gate = m.linear(m.round_cols(gate, self.rank_g), self.w_g2)
+        a, gate = u[:, self.a_col:], u[:, self.g_col:]
+        if self.w_ag2 is not None:
+            ag = m.linear(m.round_cols(a, self.rank_a + self.rank_g), self.w_ag2)   # the second steps of decay and gate: one product on the rounded first steps
+            a, gate = ag, ag[:, self.w_a2.shape[0]:]
+        else:
+            if self.w_a2 is not None:
+                a = m.linear(m.round_cols(a, self.rank_a), self.w_a2)
+            if self.w_g2 is not None:
+                gate = m.linear(m.round_cols(gate, self.rank_g), self.w_g2)
         beta = torch.empty(T, s.heads, **f32)
         dec = torch.empty(T, s.heads * self.per, **f32)
         _call("mrs_hyb_delta_prep", c, c.stride(0), u, u.stride(0), self.b_col, a, a.stride(0), self.A_log, self.dt_bias, beta, dec, T, s.heads, s.kv_heads, s.dim, self.per)
