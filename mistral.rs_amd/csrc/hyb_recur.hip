@@ -72,11 +72,9 @@ template <class T> __global__ void __launch_bounds__(256) rmsnorm_pair_kernel(co
 // c [rows, ldc]: q [G * D] | k [G * D] | v ... after convolution + SiLU; q and k are made unit vectors per head in place (x / sqrt(sum x^2 + 1e-6)), q times D^(-1/2).
 // beta [rows, H] = sigmoid(u[b_col + h]).  Decays [rows, ndec], ndec = H * per: exp(-exp(A_log[c / per]) softplus(a[c] + dt_bias[c])), the rows of `a` being a [rows, lda]
 // (per = 1: one decay per head; per = D: one per head and key channel).
-__global__ void __launch_bounds__(256) delta_prep_kernel(float *__restrict__ c, int ldc, const float *__restrict__ u, int ldu, int b_col, const float *__restrict__ a, int lda,
-                                                         const float *__restrict__ A_log, const float *__restrict__ dt_bias, float *__restrict__ beta, float *__restrict__ dec,
-                                                         int H, int G, int D, int per) {
-  const int t = blockIdx.x, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  float *cr = c + (size_t)t * ldc;
+__device__ __forceinline__ void delta_prep_row(float *cr, const float *ur, int b_col, const float *ar, const float *__restrict__ A_log, const float *__restrict__ dt_bias,
+                                               float *betar, float *decr, int H, int G, int D, int per) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const float qmul = 1.0f / sqrtf((float)D);
   for (int j = wave; j < 2 * G; j += 4) {  // head j of q | k
     float *v = cr + (size_t)j * D;
@@ -85,10 +83,64 @@ __global__ void __launch_bounds__(256) delta_prep_kernel(float *__restrict__ c, 
     const float inv = (1.0f / sqrtf(wave_sum(s) + 1e-6f)) * (j < G ? qmul : 1.0f);
     for (int d = lane; d < D; d += 64) v[d] *= inv;
   }
-  for (int h = threadIdx.x; h < H; h += 256) beta[(size_t)t * H + h] = sigmoid_f(u[(size_t)t * ldu + b_col + h]);
+  for (int h = threadIdx.x; h < H; h += 256) betar[h] = sigmoid_f(ur[b_col + h]);
   const int ndec = H * per;
-  for (int e = threadIdx.x; e < ndec; e += 256)
-    dec[(size_t)t * ndec + e] = expf(-expf(A_log[e / per]) * softplus_f(a[(size_t)t * lda + e] + dt_bias[e]));
+  for (int e = threadIdx.x; e < ndec; e += 256) decr[e] = expf(-expf(A_log[e / per]) * softplus_f(ar[e] + dt_bias[e]));
+}
+__global__ void __launch_bounds__(256) delta_prep_kernel(float *__restrict__ c, int ldc, const float *__restrict__ u, int ldu, int b_col, const float *__restrict__ a, int lda,
+                                                         const float *__restrict__ A_log, const float *__restrict__ dt_bias, float *__restrict__ beta, float *__restrict__ dec,
+                                                         int H, int G, int D, int per) {
+  const int t = blockIdx.x;
+  delta_prep_row(c + (size_t)t * ldc, u + (size_t)t * ldu, b_col, a + (size_t)t * lda, A_log, dt_bias, beta + (size_t)t * H, dec + (size_t)t * H * per, H, G, D, per);
+}
+// Steps in which every entry brings one row: the short convolution (+ SiLU) over the q | k | v columns of u with its carried taps (read, then shifted: state [slots, C,
+// taps - 1], oldest first; an entry at position 0 reads zeros) and the operands above, in one launch.  grid.y: one workgroup per q / k head (convolution, then the unit
+// vector from the workgroup's sum of squares), one per 256 value channels, and one for write strengths and decays.
+__global__ void __launch_bounds__(256) delta_step_prep_kernel(const float *__restrict__ u, int ldu, const float *__restrict__ cw, float *__restrict__ state, float *__restrict__ c,
+                                                              int ldc, int C, int taps, int b_col, const float *__restrict__ a, int lda, const float *__restrict__ A_log,
+                                                              const float *__restrict__ dt_bias, float *__restrict__ beta, float *__restrict__ dec, const int *__restrict__ seq_start,
+                                                              const int *__restrict__ seq_pos0, const int *__restrict__ seq_slot, int H, int G, int D, int per) {
+  __shared__ float red[4];
+  const int s = blockIdx.x, y = blockIdx.y, t = seq_start[s], keep = taps - 1;
+  if (seq_start[s + 1] - t != 1) return;
+  const bool carried = seq_pos0[s] > 0;
+  auto conv = [&](int ch) {
+    float *st = state + ((size_t)seq_slot[s] * C + ch) * (keep > 0 ? keep : 1);
+    const float cur = u[(size_t)t * ldu + ch];
+    float acc = 0.f, v[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      if (k >= keep) break;
+      v[k] = carried ? st[k] : 0.f;
+      acc = fmaf(cw[(size_t)ch * taps + k], v[k], acc);
+    }
+    acc = fmaf(cw[(size_t)ch * taps + keep], cur, acc);
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      if (k >= keep) break;
+      st[k] = k + 1 < keep ? v[k + 1] : cur;
+    }
+    return silu_f(acc);
+  };
+  float *cr = c + (size_t)t * ldc;
+  const int nqk = 2 * G * D, nvb = (C - nqk + 255) / 256;
+  if (y < 2 * G) {   // head y of q | k
+    float ss = 0.f;
+    for (int d = threadIdx.x; d < D; d += 256) {
+      const float v = conv(y * D + d);
+      cr[y * D + d] = v;   // re-read below by the thread that wrote it
+      ss = fmaf(v, v, ss);
+    }
+    const float inv = (1.0f / sqrtf(block_sum_256(ss, red) + 1e-6f)) * (y < G ? 1.0f / sqrtf((float)D) : 1.0f);
+    for (int d = threadIdx.x; d < D; d += 256) cr[y * D + d] *= inv;
+  } else if (y < 2 * G + nvb) {
+    const int ch = nqk + (y - 2 * G) * 256 + threadIdx.x;
+    if (ch < C) cr[ch] = conv(ch);
+  } else {
+    for (int h = threadIdx.x; h < H; h += 256) beta[(size_t)t * H + h] = sigmoid_f(u[(size_t)t * ldu + b_col + h]);
+    const int ndec = H * per;
+    for (int e = threadIdx.x; e < ndec; e += 256) dec[(size_t)t * ndec + e] = expf(-expf(A_log[e / per]) * softplus_f(a[(size_t)t * lda + e] + dt_bias[e]));
+  }
 }
 
 // ---------------------------------------------------------------------------------- delta rule: the recurrence
@@ -429,6 +481,19 @@ extern "C" int mrs_hyb_delta_prep(float *c, int ldc, const float *u, int ldu, in
   if (H <= 0 || G <= 0 || H % G || D <= 0 || (per != 1 && per != D)) return fail("mrs_hyb_delta_prep: head sizes (heads % kv_heads == 0; decays per head or per key channel)");
   hipLaunchKernelGGL(delta_prep_kernel, dim3(rows), dim3(256), 0, S_(stream), c, ldc, u, ldu, b_col, a, lda, A_log, dt_bias, beta, dec, H, G, D, per);
   return ok_or("mrs_hyb_delta_prep");
+}
+
+/* single-row steps: convolution + SiLU over the C = 2 G D + (value channels) columns of u with the slots' taps, then the operands of mrs_hyb_delta_prep, one launch */
+extern "C" int mrs_hyb_delta_step_prep(const float *u, int ldu, const float *cw, float *state, float *c, int ldc, int C, int taps, int b_col, const float *a, int lda,
+                                       const float *A_log, const float *dt_bias, float *beta, float *dec, const int *seq_start, const int *seq_pos0, const int *seq_slot,
+                                       int rows, int entries, int H, int G, int D, int per, void *stream) {
+  if (rows <= 0) return 0;
+  if (rows != entries) return fail("mrs_hyb_delta_step_prep: one row per entry");
+  if (H <= 0 || G <= 0 || H % G || D <= 0 || (per != 1 && per != D) || taps < 1 || taps > 17 || C < 2 * G * D || ldc < C) return fail("mrs_hyb_delta_step_prep: head sizes / 1 .. 17 taps");
+  if (entries > 65535 || 2 * G + (C - 2 * G * D + 255) / 256 + 1 > 65535) return fail("mrs_hyb_delta_step_prep: too many entries / heads for one launch");
+  hipLaunchKernelGGL(delta_step_prep_kernel, dim3(entries, 2 * G + (C - 2 * G * D + 255) / 256 + 1), dim3(256), 0, S_(stream), u, ldu, cw, state, c, ldc, C, taps, b_col, a, lda, A_log, dt_bias, beta, dec, seq_start, seq_pos0,
+                     seq_slot, H, G, D, per);
+  return ok_or("mrs_hyb_delta_step_prep");
 }
 
 /* c [rows, ldc] = q [G * D] | k [G * D] | v [H * Dv] (unit q / k), beta [rows, H], dec [rows, H * per] (per 1 or D), state [slots, H, D, Dv], out [rows, H * Dv].

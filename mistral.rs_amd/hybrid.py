@@ -67,6 +67,7 @@ _SIGS = {
     "mrs_hyb_route_topk_softmax": [_vp, _vp, _vp, _i, _i, _i, _i, _f, _vp, _vp, _vp],
     "mrs_hyb_rmsnorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
     "mrs_hyb_delta_prep": [_vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "mrs_hyb_delta_step_prep": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i] + [_vp] * 7 + [_i] * 6 + [_vp],
     "mrs_hyb_delta_scan": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 8 + [_vp],
     "mrs_hyb_exp_gates": [_vp, _i, _i, _i, _vp, _vp, _f] + [_vp] * 8 + [_i, _i, _i, _vp],
     "mrs_hyb_head_norm_gate": [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _vp],
@@ -77,7 +78,7 @@ _SIGS = {
     "mrs_hyb_gemv": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp],
     "mrs_hyb_gemv_act": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _l, _i, _vp, _vp, _i, _vp, _f, _f, _vp],
 }
-_RECUR = {"mrs_hyb_rmsnorm_pair", "mrs_hyb_delta_prep", "mrs_hyb_delta_scan", "mrs_hyb_exp_gates", "mrs_hyb_head_norm_gate", "mrs_hyb_norm_pair_add", "mrs_hyb_round_cols",
+_RECUR = {"mrs_hyb_rmsnorm_pair", "mrs_hyb_delta_prep", "mrs_hyb_delta_step_prep", "mrs_hyb_delta_scan", "mrs_hyb_exp_gates", "mrs_hyb_head_norm_gate", "mrs_hyb_norm_pair_add", "mrs_hyb_round_cols",
           "mrs_hyb_relu_sq"}   # launchers of csrc/hyb_recur.hip (their own error text)
 _fns: dict = {}
 _step_stream: Optional[int] = None   # the stream handle of the step in progress (looked up once per forward_batch, not once per launch)
@@ -1186,8 +1187,6 @@ class DeltaRuleMixer(_Module):
         f32 = dict(dtype=torch.float32, device=dev)
         u = m.linear(h, self.w_in)                                          # f32 [T, q | k | v | beta | a | g]
         c = torch.empty(T, self.channels, **f32)
-        _call("mrs_hyb_conv", u, u.stride(0), None, self.conv_w, None, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, c, T, b.entries, self.channels,
-              s.conv, 1)
         a, gate = u[:, self.a_col:], u[:, self.g_col:]
         if self.w_ag2 is not None:
             ag = m.linear(m.round_cols(a, self.rank_a + self.rank_g), self.w_ag2)   # the second steps of decay and gate: one product on the rounded first steps
@@ -1199,7 +1198,13 @@ class DeltaRuleMixer(_Module):
                 gate = m.linear(m.round_cols(gate, self.rank_g), self.w_g2)
         beta = torch.empty(T, s.heads, **f32)
         dec = torch.empty(T, s.heads * self.per, **f32)
-        _call("mrs_hyb_delta_prep", c, c.stride(0), u, u.stride(0), self.b_col, a, a.stride(0), self.A_log, self.dt_bias, beta, dec, T, s.heads, s.kv_heads, s.dim, self.per)
+        if T == b.entries and b.seg_rows == 1:   # every entry brings one row: convolution, tap shift and the operands in one launch
+            _call("mrs_hyb_delta_step_prep", u, u.stride(0), self.conv_w, self.conv_state, c, c.stride(0), self.channels, s.conv, self.b_col, a, a.stride(0), self.A_log,
+                  self.dt_bias, beta, dec, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, s.heads, s.kv_heads, s.dim, self.per)
+        else:
+            _call("mrs_hyb_conv", u, u.stride(0), None, self.conv_w, None, self.conv_state, b.tok_seq, b.seq_start, b.seq_pos0, b.seq_slot, c, T, b.entries, self.channels,
+                  s.conv, 1)
+            _call("mrs_hyb_delta_prep", c, c.stride(0), u, u.stride(0), self.b_col, a, a.stride(0), self.A_log, self.dt_bias, beta, dec, T, s.heads, s.kv_heads, s.dim, self.per)
         y = torch.empty(T, self.nv, **f32)
         _call("mrs_hyb_delta_scan", c, c.stride(0), beta, dec, self.state, y, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, s.heads, s.kv_heads, s.dim, s.vdim,
               self.per, 0)

@@ -341,6 +341,45 @@ def test_delta_operands(dev, H, G, D, per_channel):
     assert rel(dec.double().cpu(), want) < 2e-6
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,D,Dv,taps,per_channel", [(4, 2, 16, 8, 3, True), (3, 1, 7, 5, 1, False), (2, 2, 64, 32, 4, True), (2, 1, 130, 3, 6, False)])
+def test_single_row_steps_convolve_shift_taps_and_make_operands_in_one_launch(dev, H, G, D, Dv, taps, per_channel):
+    """three entries of one row each (one at position 0 over a NaN-filled slot, two continuing): convolution + SiLU from the slots' taps, the taps shifted, unit vectors, write
+    strengths and decays -- against the restatement; two steps in a row so that the shifted taps are read back"""
+    from mistralrs_amd.hybrid import _call
+    _lib.load("hybrid")
+    g = torch.Generator().manual_seed(D + taps)
+    per, C, keep = (D if per_channel else 1), 2 * G * D + H * Dv, max(taps - 1, 1)
+    ldu, b_col = C + H + 2, C + 1
+    cw, A_log, dtb = torch.randn(C, taps, generator=g) * 0.6, torch.randn(H, generator=g) * 0.5, torch.randn(H * per, generator=g)
+    before = [None, torch.randn(taps - 1, C, generator=g), torch.randn(taps - 1, C, generator=g)]
+    state = torch.full((4, C, keep), float("nan"), device=dev)
+    slots = (2, 0, 3)
+    for e in (1, 2):
+        if taps > 1:
+            state[slots[e]] = before[e].T.to(dev)
+    pos = [0, 9, 40]
+    for step in range(2):
+        u, a = torch.randn(3, ldu, generator=g), torch.randn(3, H * per + 3, generator=g)
+        b = _batch(dev, [(pos[e] + step, 1, slots[e]) for e in range(3)])
+        c, beta, dec = torch.empty(3, C + 2, device=dev), torch.empty(3, H, device=dev), torch.empty(3, H * per, device=dev)
+        _call("mrs_hyb_delta_step_prep", u.to(dev), ldu, cw.to(dev), state, c, C + 2, C, taps, b_col, a.to(dev), H * per + 3, A_log.to(dev), dtb.to(dev), beta, dec, b.seq_start,
+              b.seq_pos0, b.seq_slot, 3, 3, H, G, D, per)
+        for e in range(3):
+            y, before[e] = O.conv_silu(u[e:e + 1, :C].double(), cw.double(), before[e].double() if before[e] is not None else None)
+            qk = y[0, :2 * G * D].view(2 * G, D)
+            unit = qk / torch.sqrt((qk * qk).sum(-1, keepdim=True) + 1e-6)
+            unit[:G] *= D ** -0.5
+            got = c[e].double().cpu()
+            assert rel(got[:2 * G * D], unit.reshape(-1)) < 3e-6 and rel(got[2 * G * D:C], y[0, 2 * G * D:]) < 3e-6, (step, e)
+            assert rel(beta[e].double().cpu(), torch.sigmoid(u[e, b_col:b_col + H].double())) < 2e-6
+            want = torch.exp(-torch.exp(A_log.double()).repeat_interleave(per) * O.softplus(a[e, :H * per].double() + dtb.double()))
+            assert rel(dec[e].double().cpu(), want) < 2e-6
+            if taps > 1:
+                assert rel(state[slots[e]].double().cpu(), before[e].T) < 1e-7, (step, e)
+    assert bool(torch.isnan(state[1]).all())
+
+
 def _delta_rows(T, H, G, D, Dv, per, seed, slow=False):
     g = torch.Generator().manual_seed(seed)
     q, k = torch.randn(T, G, D, generator=g), torch.randn(T, G, D, generator=g)
