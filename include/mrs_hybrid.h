@@ -50,7 +50,7 @@ const char *mrs_hyb_recur_last_error();
 int mrs_hyb_rmsnorm_pair(const float *x, int ldx, const float *w1, const float *w2, void *out1, void *out2, float *out2_32, int rows, int W, float eps, int one_plus, int dtype, void *stream);
 int mrs_hyb_delta_prep(float *c, int ldc, const float *u, int ldu, int b_col, const float *a, int lda, const float *A_log, const float *dt_bias, float *beta, float *dec, int rows, int H, int G, int D, int per, void *stream);
 int mrs_hyb_delta_step_prep(const float *u, int ldu, const float *cw, float *state, float *c, int ldc, int C, int taps, int b_col, const float *a, int lda, const float *A_log, const float *dt_bias, float *beta, float *dec, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, int G, int D, int per, void *stream);
-int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, const float *dec, float *state, float *out, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, int G, int D, int Dv, int per, int lanes_per_column, void *stream);
+int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, const float *dec, float *state, float *out, const int *seq_pos0, const int *seq_slot, const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *carry, float *trans, int rows, int entries, int segments, int H, int G, int D, int Dv, int per, int lanes_per_column, void *stream);
 int mrs_hyb_exp_gates(const float *u, int ldu, int i_col, int f_col, const float *bi, const float *bf, float cap, float *m_state, float *steps, float *mbuf, float *mexp, const int *tok_seq, const int *seq_start, const int *seq_pos0, const int *seq_slot, int rows, int entries, int H, void *stream);
 int mrs_hyb_head_norm_gate(const float *y, int ldp, const float *mexp, const float *w, int w_full, const float *gate, int ldg, int gate_mode, void *out, int rows, int H, int Dv, float eps, int dtype, void *stream);
 int mrs_hyb_norm_pair_add(float *x, int ldx, const float *y1, const float *w1, const float *y2, const float *w2, int rows, int W, float eps, float c, int accumulate, void *stream);

@@ -153,33 +153,47 @@ struct DeltaArgs {
   const float *dec;    // [rows, H * per]
   float *state;        // [slots, H, D, Dv]
   float *out;          // [rows, H * Dv]
-  const int *seq_start, *seq_pos0, *seq_slot;
+  const int *seq_pos0, *seq_slot;
+  const int *seg_entry, *seg_row0, *seg_len, *ent_seg0;  // segment table: entry, first row, rows; first segment of every entry (+ the total)
+  float *carry;        // [segments, H, D, Dv]: a segment's end state from zero, then the state the next segment starts from
+  float *trans;        // [segments, H, D, D]: what a segment does to a state it is handed (the product of its rows' transitions)
   int ldc, H, G, D, Dv, per;
 };
-template <int R, int K, bool VEC, int MAXREG> __global__ void __launch_bounds__(512) delta_scan_kernel(DeltaArgs a, int rowpad, int TC) {
+// The recurrence is linear in S: a row maps S -> (I - beta k k^T) diag(g) S + beta k v^T, the matrix in front being the same for every value column.  A long portion can
+// therefore run its segments side by side like the other scans of this library:
+//   A  every segment but an entry's last, from the state [0 | I] with the values [v | 0]: D further columns carry the identity through the same steps, so the segment leaves its
+//      end state from zero L_k and its transition P_k                                                                                      (parallel over segments; LOCAL)
+//   B  init_(k+1) = P_k init_k + L_k, init_0 = the slot's state (zero for an entry that starts at position 0)                              (delta_carry_kernel)
+//   C  every segment from its init state: the outputs; an entry's last segment leaves the slot's new state                                (parallel over segments)
+// An entry of one segment is pass C alone; the host runs A and B only when the step's entries alone would leave most of the chip idle.
+template <int R, int K, bool VEC, int MAXREG, bool LOCAL> __global__ void __launch_bounds__(512) delta_scan_kernel(DeltaArgs a, int rowpad, int TC) {
   extern __shared__ __attribute__((aligned(16))) float sm[];  // [2][TC][rowpad]: k [D] | q [D] | decay [per] (padded to 4) | v [Dv] | beta
   constexpr int PT = 64 / R;
   const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, r = lane % R, p = (blockIdx.x * (nthr >> 6) + wave) * PT + lane / R;
-  const int h = blockIdx.y, s = blockIdx.z;
-  const int r0 = a.seq_start[s], len = a.seq_start[s + 1] - r0;
-  if (len <= 0) return;
+  const int h = blockIdx.y, z = blockIdx.z;
+  const int s = a.seg_entry[z], r0 = a.seg_row0[z], len = a.seg_len[z];
+  const bool first = z == a.ent_seg0[s], last = z == a.ent_seg0[s + 1] - 1;
+  if (len <= 0 || (LOCAL && last)) return;
   const int D = a.D, Dv = a.Dv, per = a.per, g = h / (a.H / a.G);
-  const bool live = p < Dv;
-  const int pc = live ? p : Dv - 1;
+  const int ncol = LOCAL ? Dv + D : Dv;
+  const bool live = p < ncol;
+  const int pa = live ? p : ncol - 1;
+  const bool ident = LOCAL && pa >= Dv;      // a column of the identity: no value, no output
+  const int pc = ident ? 0 : pa, idc = pa - Dv;
   int nk = D - r * K;
   nk = nk < 0 ? 0 : (nk > K ? K : nk);
   float *st = a.state + ((size_t)a.seq_slot[s] * a.H + h) * D * Dv;
-  const bool carried = a.seq_pos0[s] > 0;
+  const float *init = LOCAL ? nullptr : (first ? (a.seq_pos0[s] > 0 ? st : nullptr) : a.carry + ((size_t)(z - 1) * a.H + h) * D * Dv);
   float S[K];
 #pragma unroll
-  for (int k = 0; k < K; ++k) S[k] = (k < nk && carried) ? st[(size_t)(r * K + k) * Dv + pc] : 0.f;
+  for (int k = 0; k < K; ++k) S[k] = k < nk ? (LOCAL ? ((ident && r * K + k == idc) ? 1.0f : 0.f) : (init ? init[(size_t)(r * K + k) * Dv + pc] : 0.f)) : 0.f;
   const int perp = (per + 3) & ~3, o_q = D, o_g = 2 * D, o_v = 2 * D + perp, o_b = o_v + Dv, rowlen = o_b + 1, stage = TC * rowpad;
   const int qcol = g * D, kcol = a.G * D + g * D, vcol = 2 * a.G * D + h * Dv;
   // this lane's operands of one staged row: k, decay and q of its K state rows (zeros / ones past the key size), the column's value and the write strength
   constexpr bool PREFETCH = K <= 16;
   const int base = nk ? r * K : 0;
   auto ops = [&](const float *row, float *kv, float *gv, float *qv, float *sv) {
-    sv[0] = row[o_v + pc];
+    sv[0] = ident ? 0.f : row[o_v + pc];
     sv[1] = row[o_b];
     const float g1 = row[o_g];
     if (VEC) {
@@ -274,9 +288,11 @@ template <int R, int K, bool VEC, int MAXREG> __global__ void __launch_bounds__(
           o1 = fmaf(S[k + 1], qc[k + 1], o1);
         }
       }
-      const float o = group_sum<R>(o0 + o1);
-      if (r == 0 && live) *op = o;
-      op += ostep;
+      if (!LOCAL) {
+        const float o = group_sum<R>(o0 + o1);
+        if (r == 0 && live) *op = o;
+        op += ostep;
+      }
     };
     if (PREFETCH) {
       ops(cur, ka, ga, qa, sa);
@@ -297,10 +313,50 @@ template <int R, int K, bool VEC, int MAXREG> __global__ void __launch_bounds__(
     if (more) put(sm + (flip ^ 1) * stage);
     __syncthreads();
   }
-  if (live)
+  if (LOCAL) {
+    float *dst = ident ? a.trans + ((size_t)z * a.H + h) * D * D + idc : a.carry + ((size_t)z * a.H + h) * D * Dv + pc;
+    const int ld = ident ? D : Dv;
+    if (live)
+#pragma unroll
+      for (int k = 0; k < K; ++k)
+        if (k < nk) dst[(size_t)(r * K + k) * ld] = S[k];
+  } else if (live && last) {
 #pragma unroll
     for (int k = 0; k < K; ++k)
       if (k < nk) st[(size_t)(r * K + k) * Dv + p] = S[k];
+  }
+}
+// pass B: one workgroup per (4 value columns, head, entry); thread n owns state row n of the four columns.  Serial over the entry's segments:
+// new[n][:] = sum_m P[n][m] cur[m][:] + L[n][:], cur in LDS; carry[z] (L on entry) leaves as the state segment z + 1 starts from.
+__global__ void __launch_bounds__(256) delta_carry_kernel(DeltaArgs a) {
+  __shared__ __attribute__((aligned(16))) float cur[256][4];
+  const int n = threadIdx.x, p0 = blockIdx.x * 4, h = blockIdx.y, s = blockIdx.z;
+  const int z0 = a.ent_seg0[s], z1 = a.ent_seg0[s + 1], D = a.D, Dv = a.Dv;
+  if (z1 - z0 < 2) return;
+  const float *st = a.state + ((size_t)a.seq_slot[s] * a.H + h) * D * Dv;
+  const bool carried = a.seq_pos0[s] > 0;
+  float v[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) v[j] = (carried && n < D && p0 + j < Dv) ? st[(size_t)n * Dv + p0 + j] : 0.f;
+  for (int z = z0; z < z1 - 1; ++z) {
+    __syncthreads();   // the previous round has read cur
+    if (n < D) *(float4 *)cur[n] = make_float4(v[0], v[1], v[2], v[3]);
+    __syncthreads();
+    if (n < D) {
+      const float *P = a.trans + (((size_t)z * a.H + h) * D + n) * D;
+      float *L = a.carry + (((size_t)z * a.H + h) * D + n) * Dv + p0;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) v[j] = p0 + j < Dv ? L[j] : 0.f;
+      for (int m = 0; m < D; ++m) {
+        const float pm = P[m];
+        const float4 c4 = *(const float4 *)cur[m];
+        v[0] = fmaf(pm, c4.x, v[0]); v[1] = fmaf(pm, c4.y, v[1]); v[2] = fmaf(pm, c4.z, v[2]); v[3] = fmaf(pm, c4.w, v[3]);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (p0 + j < Dv) L[j] = v[j];
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------------- exponential gates with a running stabiliser
@@ -497,41 +553,58 @@ extern "C" int mrs_hyb_delta_step_prep(const float *u, int ldu, const float *cw,
 }
 
 /* c [rows, ldc] = q [G * D] | k [G * D] | v [H * Dv] (unit q / k), beta [rows, H], dec [rows, H * per] (per 1 or D), state [slots, H, D, Dv], out [rows, H * Dv].
- * lanes_per_column 0: chosen from the step's parallelism (4 when entries x heads x columns fill the chip, else 16: shorter serial chains). */
-extern "C" int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, const float *dec, float *state, float *out, const int *seq_start, const int *seq_pos0,
-                                  const int *seq_slot, int rows, int entries, int H, int G, int D, int Dv, int per, int lanes_per_column, void *stream) {
-  if (rows <= 0 || entries <= 0) return 0;
+ * Segment table as for the other scans.  carry [segments, H, D, Dv] and trans [segments, H, D, D] (nullable scratch): with them, a step whose entries alone would leave most of
+ * the chip idle runs the segments of its long portions side by side (three passes); without them, or when entries x heads x columns fill the chip, every entry is one chain.
+ * lanes_per_column 0: chosen from the step's parallelism (4, or 16 for shorter serial chains). */
+extern "C" int mrs_hyb_delta_scan(const float *c, int ldc, const float *beta, const float *dec, float *state, float *out, const int *seq_pos0, const int *seq_slot,
+                                  const int *seg_entry, const int *seg_row0, const int *seg_len, const int *ent_seg0, float *carry, float *trans, int rows, int entries,
+                                  int segments, int H, int G, int D, int Dv, int per, int lanes_per_column, void *stream) {
+  if (rows <= 0 || entries <= 0 || segments <= 0) return 0;
   if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0 || (per != 1 && per != D)) return fail("mrs_hyb_delta_scan: head sizes (heads % kv_heads == 0; decays per head or per key channel)");
   if (D > 256) return fail("mrs_hyb_delta_scan: key size above 256");
-  if (entries > 65535 || H > 65535) return fail("mrs_hyb_delta_scan: more than 65535 entries or heads");
+  if (entries > 65535 || segments > 65535 || H > 65535) return fail("mrs_hyb_delta_scan: more than 65535 entries, segments or heads");
   if (ldc < 2 * G * D + H * Dv) return fail("mrs_hyb_delta_scan: rows shorter than q | k | v");
-  DeltaArgs a{c, beta, dec, state, out, seq_start, seq_pos0, seq_slot, ldc, H, G, D, Dv, per};
+  if (segments > entries && (!carry || !trans)) return fail("mrs_hyb_delta_scan: segmented entries need the carry scratch");
+  DeltaArgs a{c, beta, dec, state, out, seq_pos0, seq_slot, seg_entry, seg_row0, seg_len, ent_seg0, carry, trans, ldc, H, G, D, Dv, per};
+  const bool split = segments > entries;
+  const long long par = (long long)segments * H * ((Dv + 15) / 16);   // waves at four lanes per column
   int R = lanes_per_column;
-  if (R != 4 && R != 16) R = ((long long)entries * H * ((Dv + 15) / 16) >= 2048 || D < 64) ? 4 : 16;
+  if (R != 4 && R != 16) R = (par >= 2048 || D < 64) ? 4 : 16;
   const int PT = 64 / R;
   const int perp = (per + 3) & ~3, rowlen = 2 * D + perp + Dv + 1, rowpad = (rowlen + 3) & ~3;
   constexpr int MAXREG = 12, TC_MAX = 16;
-  // waves for the columns; waves whose registers can stage eight rows of operands at a time (a stage must outlast the latency of the loads for the next one)
-  const int nw_all = (Dv + PT - 1) / PT, nw_stage = (8 * rowpad + MAXREG * 64 - 1) / (MAXREG * 64);
-  int nw = nw_all > 8 ? 8 : nw_all;   // (four-wave workgroups, one chain per SIMD, measured no faster: the chain is bound by its own instruction count)
-  const int nblk = (nw_all + nw - 1) / nw;
-  if (nw < nw_stage) nw = nw_stage > 8 ? 8 : nw_stage;  // few value columns next to long keys: further waves only help to stage (their columns lie past Dv and are never written)
-  int TC = (MAXREG * 64 * nw) / rowpad;
-  TC = TC > TC_MAX ? TC_MAX : TC;
-  if (TC > 65536 / (8 * rowpad)) TC = 65536 / (8 * rowpad);
-  if (TC < 1) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers / 64 KB of LDS");
-  const size_t lds = (size_t)2 * TC * rowpad * 4;
   const bool vec = D % 4 == 0;
-  dim3 grid(nblk, H, entries), block(64 * nw);
-#define MRS_DELTA_(R_, K_, V_) hipLaunchKernelGGL((delta_scan_kernel<R_, K_, V_, MAXREG>), grid, block, lds, S_(stream), a, rowpad, TC)
+  auto launch = [&](bool local) {
+    const int ncol = local ? Dv + D : Dv;
+    // waves for the columns; waves whose registers can stage eight rows of operands at a time (a stage must outlast the latency of the loads for the next one)
+    const int nw_all = (ncol + PT - 1) / PT, nw_stage = (8 * rowpad + MAXREG * 64 - 1) / (MAXREG * 64);
+    int nw = nw_all > 8 ? 8 : nw_all;   // (four-wave workgroups, one chain per SIMD, measured no faster: the chain is bound by its own instruction count)
+    const int nblk = (nw_all + nw - 1) / nw;
+    if (nw < nw_stage) nw = nw_stage > 8 ? 8 : nw_stage;  // few value columns next to long keys: further waves only help to stage (their columns lie past the last one and are never written)
+    int TC = (MAXREG * 64 * nw) / rowpad;
+    TC = TC > TC_MAX ? TC_MAX : TC;
+    if (TC > 65536 / (8 * rowpad)) TC = 65536 / (8 * rowpad);
+    if (TC < 1) return fail("mrs_hyb_delta_scan: a row of operands does not fit the staging registers / 64 KB of LDS");
+    const size_t lds = (size_t)2 * TC * rowpad * 4;
+    dim3 grid(nblk, H, segments), block(64 * nw);
+#define MRS_DELTA__(R_, K_, V_, L_) hipLaunchKernelGGL((delta_scan_kernel<R_, K_, V_, MAXREG, L_>), grid, block, lds, S_(stream), a, rowpad, TC)
+#define MRS_DELTA_(R_, K_, V_) do { if (local) MRS_DELTA__(R_, K_, V_, true); else MRS_DELTA__(R_, K_, V_, false); } while (0)
 #define MRS_DELTA(R_, K_) do { if (vec) MRS_DELTA_(R_, K_, true); else MRS_DELTA_(R_, K_, false); } while (0)
-  if (R == 4) {
-    if (D <= 32) MRS_DELTA(4, 8); else if (D <= 64) MRS_DELTA(4, 16); else if (D <= 128) MRS_DELTA(4, 32); else MRS_DELTA(4, 64);
-  } else {
-    if (D <= 64) MRS_DELTA(16, 4); else if (D <= 128) MRS_DELTA(16, 8); else MRS_DELTA(16, 16);
-  }
+    if (R == 4) {
+      if (D <= 32) MRS_DELTA(4, 8); else if (D <= 64) MRS_DELTA(4, 16); else if (D <= 128) MRS_DELTA(4, 32); else MRS_DELTA(4, 64);
+    } else {
+      if (D <= 64) MRS_DELTA(16, 4); else if (D <= 128) MRS_DELTA(16, 8); else MRS_DELTA(16, 16);
+    }
 #undef MRS_DELTA
 #undef MRS_DELTA_
+#undef MRS_DELTA__
+    return 0;
+  };
+  if (split) {
+    if (launch(true)) return 1;
+    hipLaunchKernelGGL(delta_carry_kernel, dim3((Dv + 3) / 4, H, entries), dim3(256), 0, S_(stream), a);
+  }
+  if (launch(false)) return 1;
   return ok_or("mrs_hyb_delta_scan");
 }
 

@@ -68,7 +68,7 @@ _SIGS = {
     "mrs_hyb_rmsnorm_pair": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _i, _f, _i, _i, _vp],
     "mrs_hyb_delta_prep": [_vp, _i, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "mrs_hyb_delta_step_prep": [_vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _vp, _i] + [_vp] * 7 + [_i] * 6 + [_vp],
-    "mrs_hyb_delta_scan": [_vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp] + [_i] * 8 + [_vp],
+    "mrs_hyb_delta_scan": [_vp, _i] + [_vp] * 12 + [_i] * 9 + [_vp],
     "mrs_hyb_exp_gates": [_vp, _i, _i, _i, _vp, _vp, _f] + [_vp] * 8 + [_i, _i, _i, _vp],
     "mrs_hyb_head_norm_gate": [_vp, _i, _vp, _vp, _i, _vp, _i, _i, _vp, _i, _i, _i, _f, _i, _vp],
     "mrs_hyb_norm_pair_add": [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _f, _f, _i, _vp],
@@ -120,6 +120,16 @@ class RaggedBatch:
     seg_rows: int = 0                          # rows of the longest segment (1: every entry brings one decoded token)
     host_blocks: Optional[List[Sequence[int]]] = None   # every entry's block ids covering its last position (host copy; `build` keeps it)
     _context: Optional[tuple] = None
+    _entries: Optional[tuple] = None
+
+    def entry_table(self):
+        """A segment table with ONE segment per entry, however long: (seg_entry, seg_row0, seg_len, ent_seg0) for a scan that runs every entry as one chain."""
+        if self.segments == self.entries:
+            return self.seg_entry, self.seg_row0, self.seg_len, self.ent_seg0
+        if self._entries is None:
+            iota = torch.arange(self.entries + 1, dtype=torch.int32, device=self.tokens.device)
+            self._entries = (iota[:-1], self.seq_start[:-1], (self.seq_start[1:] - self.seq_start[:-1]).contiguous(), iota)
+        return self._entries
 
     def context_blocks(self):
         """The blocks that hold the batch's whole contexts, renumbered densely: (tables i32 [entries, max_blocks] of dense ids, source i32 [n] = the pool block behind
@@ -1134,6 +1144,9 @@ class DeltaRuleMixer(_Module):
     head or per (head, key channel).  Per head the f32 state S [dim, vdim] (carried per slot): S <- diag(g) S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q.
     o / rms(o) per head times the weight `norm` [vdim] times the gate, then the output projection.  Head h reads q / k head h // (heads / kv_heads)."""
 
+    CHAIN_WAVES = int(os.environ.get("MRS_DELTA_CHAIN_WAVES", "256"))   # entries x heads x (value size / 16) below this: long portions run their segments in parallel
+    LANES = int(os.environ.get("MRS_DELTA_LANES", "0"))                 # lanes per state column (4 | 16); 0: the launcher chooses
+
     def __init__(self, model, spec: DeltaRuleSpec, prefix: str):
         super().__init__(model)
         self.s, self.p = spec, prefix
@@ -1206,8 +1219,15 @@ class DeltaRuleMixer(_Module):
                   s.conv, 1)
             _call("mrs_hyb_delta_prep", c, c.stride(0), u, u.stride(0), self.b_col, a, a.stride(0), self.A_log, self.dt_bias, beta, dec, T, s.heads, s.kv_heads, s.dim, self.per)
         y = torch.empty(T, self.nv, **f32)
-        _call("mrs_hyb_delta_scan", c, c.stride(0), beta, dec, self.state, y, b.seq_start, b.seq_pos0, b.seq_slot, T, b.entries, s.heads, s.kv_heads, s.dim, s.vdim,
-              self.per, 0)
+        if b.segments > b.entries and b.entries * s.heads * -(-s.vdim // 16) < self.CHAIN_WAVES:
+            # long portions in a step that would leave most of the chip idle: their segments side by side (end states from zero and transitions, a carry, then the outputs)
+            table, nseg = (b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0), b.segments
+            carry = torch.empty(nseg, s.heads, s.dim, s.vdim, **f32)
+            trans = torch.empty(nseg, s.heads, s.dim, s.dim, **f32)
+        else:
+            table, nseg, carry, trans = b.entry_table(), b.entries, None, None   # every entry one chain; entries x heads x columns fill the chip (or all are short)
+        _call("mrs_hyb_delta_scan", c, c.stride(0), beta, dec, self.state, y, b.seq_pos0, b.seq_slot, *table, carry, trans, T, b.entries, nseg, s.heads, s.kv_heads, s.dim,
+              s.vdim, self.per, self.LANES)
         o = torch.empty(T, self.nv, dtype=m.torch_dtype, device=dev)
         _call("mrs_hyb_head_norm_gate", y, s.vdim, None, self.norm, 0, gate, gate.stride(0), 1 if self.w_g2 is not None else 2, o, T, s.heads, s.vdim, m.spec.eps, m.dt)
         m.linear(o, self.w_o, out=x, accumulate=accumulate)

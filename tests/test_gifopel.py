@@ -391,15 +391,17 @@ def _delta_rows(T, H, G, D, Dv, per, seed, slow=False):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("segmented", [False, True], ids=["chains", "segments"])
 @pytest.mark.parametrize("H,G,D,Dv,per_channel,lanes", [(4, 2, 16, 8, True, 0), (2, 1, 32, 32, False, 4), (2, 2, 64, 16, True, 16), (3, 1, 7, 5, True, 0), (1, 1, 130, 3, False, 16),
                                                          (2, 2, 128, 40, True, 4), (2, 1, 256, 130, True, 0), (5, 5, 1, 1, False, 0)])
-def test_delta_recurrence_over_portions_single_rows_and_reused_slots(dev, H, G, D, Dv, per_channel, lanes):
-    """three sequences through slots that hold a former owner's numbers: portions of several sizes beside single rows, every row against the restatement on the whole sequence"""
+def test_delta_recurrence_over_portions_single_rows_and_reused_slots(dev, H, G, D, Dv, per_channel, lanes, segmented):
+    """three sequences through slots that hold a former owner's numbers: portions of several sizes (some longer than two segments of 64 rows) beside single rows, every entry
+    as one chain or its segments side by side, every row against the restatement on the whole sequence"""
     from mistralrs_amd.hybrid import _call
     _lib.load("hybrid")
     per = D if per_channel else 1
-    lens = (50, 21, 9)
-    seqs = [_delta_rows(n, H, G, D, Dv, per, 10 * D + k) for k, n in enumerate(lens)]
+    lens = (250, 151, 9)
+    seqs = [_delta_rows(n, H, G, D, Dv, per, 10 * D + k, slow=k == 0) for k, n in enumerate(lens)]   # the longest one decays slowly: what a segment is handed matters
     rep = H // G
     want = []
     for q, k, v, beta, dec in seqs:
@@ -423,7 +425,12 @@ def test_delta_recurrence_over_portions_single_rows_and_reused_slots(dev, H, G, 
         beta = torch.cat([seqs[j][3][at[j]:at[j] + n] for j, n in parts]).to(dev)
         dec = torch.cat([seqs[j][4][at[j]:at[j] + n].reshape(n, -1) for j, n in parts]).to(dev)
         y = torch.empty(c.shape[0], H * Dv, device=dev)
-        _call("mrs_hyb_delta_scan", c, ldc, beta, dec, state, y, b.seq_start, b.seq_pos0, b.seq_slot, c.shape[0], len(parts), H, G, D, Dv, per, lanes)
+        if segmented:
+            carry, trans = torch.empty(b.segments, H, D, Dv, device=dev), torch.empty(b.segments, H, D, D, device=dev)
+            _call("mrs_hyb_delta_scan", c, ldc, beta, dec, state, y, b.seq_pos0, b.seq_slot, b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0, carry, trans, c.shape[0], len(parts),
+                  b.segments, H, G, D, Dv, per, lanes)
+        else:
+            _call("mrs_hyb_delta_scan", c, ldc, beta, dec, state, y, b.seq_pos0, b.seq_slot, *b.entry_table(), None, None, c.shape[0], len(parts), len(parts), H, G, D, Dv, per, lanes)
         r = 0
         for j, n in parts:
             got[j].append(y[r:r + n].double().cpu())
@@ -433,10 +440,11 @@ def test_delta_recurrence_over_portions_single_rows_and_reused_slots(dev, H, G, 
     run([1, 1, 1])
     run([2, 5, 3])
     run([1, 0, 2])
-    run([16, 13, 3])
+    run([150, 64, 3])      # three segments (64 + 64 + 22) beside exactly one beside a short one
+    run([66, 79, 0])
     assert at == list(lens)
     for j in range(3):
-        assert rel(torch.cat(got[j]), want[j]) < 1e-5, j
+        assert rel(torch.cat(got[j]), want[j]) < 2e-5, j
     assert bool((state[2] == 1e6).all()) and bool(torch.isnan(state[1]).all())
 
 
@@ -465,8 +473,9 @@ def test_delta_state_keeps_a_planted_pair_for_hundreds_of_rows_and_replaces_it(d
     for n in (63, 1, 64, 2, 65, 1, 1, 130, 3, 70):
         b = _batch(dev, [(at, n, 1)])
         y = torch.empty(n, H * Dv, device=dev)
-        _call("mrs_hyb_delta_scan", c[at:at + n].to(dev), ldc, beta[at:at + n].to(dev), dec[at:at + n].reshape(n, -1).to(dev), state, y, b.seq_start, b.seq_pos0, b.seq_slot, n, 1,
-              H, H, D, Dv, D, 0)
+        carry, trans = torch.empty(b.segments, H, D, Dv, device=dev), torch.empty(b.segments, H, D, D, device=dev)
+        _call("mrs_hyb_delta_scan", c[at:at + n].to(dev), ldc, beta[at:at + n].to(dev), dec[at:at + n].reshape(n, -1).to(dev), state, y, b.seq_pos0, b.seq_slot, b.seg_entry,
+              b.seg_row0, b.seg_len, b.ent_seg0, carry, trans, n, 1, b.segments, H, H, D, Dv, D, 0)
         outs.append(y.double().cpu())
         at += n
     y = torch.cat(outs)[:, :Dv]
