@@ -1182,11 +1182,12 @@ def gifopel_leg(a, dev):
                 sp = mx.s
                 c = torch.randn(T, mx.channels, **f32) * 0.1
                 beta, dec, yy = torch.rand(T, sp.heads, **f32), 1 - 0.1 * torch.rand(T, sp.heads * mx.per, **f32), torch.empty(T, mx.nv, **f32)
-                if b.segments > b.entries and b.entries * sp.heads * -(-sp.vdim // 16) < mx.CHAIN_WAVES:   # the mixer's own choice: segments side by side, or one chain per entry
-                    table, nseg = (b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0), b.segments
-                    cy, tr = torch.empty(nseg, sp.heads, sp.dim, sp.vdim, **f32), torch.empty(nseg, sp.heads, sp.dim, sp.dim, **f32)
-                else:
-                    table, nseg, cy, tr = b.entry_table(), b.entries, None, None
+                table, nseg, cy, tr = b.entry_table(), b.entries, None, None
+                if b.seg_rows > 1 and b.entries * sp.heads * -(-sp.vdim // 16) < mx.CHAIN_WAVES:   # the mixer's own choice: segments side by side, or one chain per entry
+                    *cut, n = b.segment_table(mx.SEGMENT)
+                    if n > b.entries:
+                        table, nseg = cut, n
+                        cy, tr = torch.empty(nseg, sp.heads, sp.dim, sp.vdim, **f32), torch.empty(nseg, sp.heads, sp.dim, sp.dim, **f32)
                 t_new = timed(lambda: _call("mrs_hyb_delta_scan", c, mx.channels, beta, dec, mx.state, yy, b.seq_pos0, b.seq_slot, *table, cy, tr, T, b.entries, nseg, sp.heads,
                                             sp.kv_heads, sp.dim, sp.vdim, mx.per, mx.LANES), 5)
                 t_old = timed(ssd(b, o2), 5)

@@ -119,8 +119,33 @@ class RaggedBatch:
     ent_seg0: Optional[torch.Tensor] = None    # i32 [entries + 1]  first segment of every entry, then the total
     seg_rows: int = 0                          # rows of the longest segment (1: every entry brings one decoded token)
     host_blocks: Optional[List[Sequence[int]]] = None   # every entry's block ids covering its last position (host copy; `build` keeps it)
+    host_lens: Optional[List[int]] = None               # rows of every entry (host copy; `build` keeps it)
     _context: Optional[tuple] = None
     _entries: Optional[tuple] = None
+    _long: Optional[dict] = None
+
+    def segment_table(self, rows: int):
+        """The batch's entries cut into segments of at most `rows` rows (another cut than SEGMENT, for a scan whose pass between the segments is dear):
+        (seg_entry, seg_row0, seg_len, ent_seg0, segments)."""
+        if rows == RaggedBatch.SEGMENT or self.host_lens is None:
+            return self.seg_entry, self.seg_row0, self.seg_len, self.ent_seg0, self.segments
+        if self._long is None:
+            self._long = {}
+        if rows not in self._long:
+            nseg = sum(max(1, -(-n // rows)) for n in self.host_lens)
+            t = np.zeros(3 * nseg + self.entries + 1, dtype=np.int32)
+            sge, sgr, sgl, es0 = t[:nseg], t[nseg:2 * nseg], t[2 * nseg:3 * nseg], t[3 * nseg:]
+            z = r = 0
+            for s, n in enumerate(self.host_lens):
+                es0[s] = z
+                for a0 in range(0, max(n, 1), rows):
+                    sge[z], sgr[z], sgl[z] = s, r + a0, min(rows, n - a0)
+                    z += 1
+                r += n
+            es0[self.entries] = z
+            d = torch.from_numpy(t).to(self.tokens.device)
+            self._long[rows] = (d[:nseg], d[nseg:2 * nseg], d[2 * nseg:3 * nseg], d[3 * nseg:], nseg)
+        return self._long[rows]
 
     def entry_table(self):
         """A segment table with ONE segment per entry, however long: (seg_entry, seg_row0, seg_len, ent_seg0) for a scan that runs every entry as one chain."""
@@ -203,7 +228,7 @@ class RaggedBatch:
             dv.append(dev_ints[o:o + n])
             o += n
         return RaggedBatch(T, S, mb, dv[0], dv[1], dv[2], dv[3], dv[4], dv[5], dv[6].view(S, mb), torch.from_numpy(slots).to(device),
-                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10], max(1, min(L, max(lens, default=1))), host_blocks)
+                           torch.tensor(want, dtype=torch.int32, device=device), nseg, dv[7], dv[8], dv[9], dv[10], max(1, min(L, max(lens, default=1))), host_blocks, lens)
 
 
 # ------------------------------------------------------------------------------------------------------------------ layer descriptions
@@ -1146,6 +1171,7 @@ class DeltaRuleMixer(_Module):
 
     CHAIN_WAVES = int(os.environ.get("MRS_DELTA_CHAIN_WAVES", "256"))   # entries x heads x (value size / 16) below this: long portions run their segments in parallel
     LANES = int(os.environ.get("MRS_DELTA_LANES", "0"))                 # lanes per state column (4 | 16); 0: the launcher chooses
+    SEGMENT = int(os.environ.get("MRS_DELTA_SEGMENT", "128"))           # rows per segment of that form: the carry between segments costs dim^2 vdim per segment
 
     def __init__(self, model, spec: DeltaRuleSpec, prefix: str):
         super().__init__(model)
@@ -1219,13 +1245,14 @@ class DeltaRuleMixer(_Module):
                   s.conv, 1)
             _call("mrs_hyb_delta_prep", c, c.stride(0), u, u.stride(0), self.b_col, a, a.stride(0), self.A_log, self.dt_bias, beta, dec, T, s.heads, s.kv_heads, s.dim, self.per)
         y = torch.empty(T, self.nv, **f32)
-        if b.segments > b.entries and b.entries * s.heads * -(-s.vdim // 16) < self.CHAIN_WAVES:
+        table, nseg, carry, trans = b.entry_table(), b.entries, None, None      # every entry one chain: entries x heads x columns fill the chip, or all are short
+        if b.seg_rows > 1 and b.entries * s.heads * -(-s.vdim // 16) < self.CHAIN_WAVES:
             # long portions in a step that would leave most of the chip idle: their segments side by side (end states from zero and transitions, a carry, then the outputs)
-            table, nseg = (b.seg_entry, b.seg_row0, b.seg_len, b.ent_seg0), b.segments
-            carry = torch.empty(nseg, s.heads, s.dim, s.vdim, **f32)
-            trans = torch.empty(nseg, s.heads, s.dim, s.dim, **f32)
-        else:
-            table, nseg, carry, trans = b.entry_table(), b.entries, None, None   # every entry one chain; entries x heads x columns fill the chip (or all are short)
+            *cut, n = b.segment_table(self.SEGMENT)
+            if n > b.entries:
+                table, nseg = cut, n
+                carry = torch.empty(nseg, s.heads, s.dim, s.vdim, **f32)
+                trans = torch.empty(nseg, s.heads, s.dim, s.dim, **f32)
         _call("mrs_hyb_delta_scan", c, c.stride(0), beta, dec, self.state, y, b.seq_pos0, b.seq_slot, *table, carry, trans, T, b.entries, nseg, s.heads, s.kv_heads, s.dim,
               s.vdim, self.per, self.LANES)
         o = torch.empty(T, self.nv, dtype=m.torch_dtype, device=dev)
