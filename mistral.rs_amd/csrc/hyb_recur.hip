@@ -4,7 +4,9 @@
 //
 //   norm pair            one root mean square, two weights: the inputs of a layer's mixer and feed-forward in one pass over the residual row
 //   delta prep           unit-length queries and keys per head, write strengths, decays per head or per (head, key channel)
+//   delta step prep      the same behind the short convolution and its tap shift, for steps of single rows: one launch
 //   delta scan           S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q            (f32 state [slot, head, D, Dv])
+//                        every entry one chain, or the segments of long portions side by side (end states and transitions from zero | identity, a carry, the outputs)
 //   exponential gates    capped log gates, the running maximum m, the step values e^{i - m'}, e^{f + m - m'} and e^{-m'} of every row
 //   head norm + gate     per-head output norm (optionally behind a normaliser column), shared or full weight, sigmoid / SiLU gate, rounded once for the out-projection
 //   normed average       x (+)= c (y1 / rms(y1) w1 + y2 / rms(y2) w2)
